@@ -473,6 +473,60 @@ __global__ void glu_kernel(const float* __restrict__ y, void* __restrict__ out, 
   Act<AF32>::store(static_cast<typename Act<AF32>::type*>(out), i, (kind == 0 ? fmaxf(g, 0.f) : siluf_(g)) * u);
 }
 
+// ---------------------------------------------------------------- residual step with a Dynamic Tanh norm
+// x += mult * y (when y is given); then, when an output is given, out = tanh(alpha * x) * w + b (w given) or
+// out = x (no w: the stream itself in the activation type). Nothing is reduced over a row, so a thread owns V
+// neighbouring coordinates (V = 4 when the width allows 16-byte accesses). ``ldo``: row stride of ``out``
+// (a column block of a wider matrix).
+template <bool AF32, int V>
+__global__ void add_dyt_kernel(float* __restrict__ x, const float* __restrict__ y, float mult, float alpha,
+                               const float* __restrict__ w, const float* __restrict__ b, void* __restrict__ out, int ldo,
+                               long long total, int d) {
+  const long long i = (static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x) * V;
+  if (i >= total) return;
+  const long long t = i / d;
+  const int c = static_cast<int>(i - t * d);
+  float v[V];
+#pragma unroll
+  for (int e = 0; e < V; ++e) v[e] = x[i + e];
+  if (y != nullptr) {
+#pragma unroll
+    for (int e = 0; e < V; ++e) {
+      v[e] += mult * y[i + e];
+      x[i + e] = v[e];
+    }
+  }
+  if (out == nullptr) return;
+  typename Act<AF32>::type* o = static_cast<typename Act<AF32>::type*>(out);
+#pragma unroll
+  for (int e = 0; e < V; ++e) {
+    const float r = w != nullptr ? tanhf(alpha * v[e]) * w[c + e] + b[c + e] : v[e];
+    Act<AF32>::store(o, static_cast<size_t>(t) * ldo + c + e, r);
+  }
+}
+
+// Clamped gated unit of y = (gate | up) columns of an fp32 matrix: g = min(s * gate, limit),
+// u = clamp(s * up, -limit, limit), out = g * sigmoid(slope * g) * (u + shift). Row r of the work list is
+// row slot_of[r] of y and of out with s = wts[r] (expert-sorted rows of a routed feed-forward, whose
+// weight scales the expert's INPUT: the products are linear, so the scale is applied to them), or row r
+// itself with s = 1 when no list is given.
+template <bool AF32>
+__global__ void glu_clamped_kernel(const float* __restrict__ y, int ld, int col_gate, int col_up, int n, float limit,
+                                   float slope, float shift, const int32_t* __restrict__ slot_of,
+                                   const float* __restrict__ wts, void* __restrict__ out, long long total) {
+  const long long i = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i >= total) return;
+  const long long r = i / n;
+  const int c = static_cast<int>(i - r * n);
+  const long long p = slot_of != nullptr ? slot_of[r] : r;
+  const float s = wts != nullptr ? wts[r] : 1.f;
+  const float* row = y + p * ld;
+  const float g = fminf(row[col_gate + c] * s, limit);
+  const float u = fminf(fmaxf(row[col_up + c] * s, -limit), limit);
+  Act<AF32>::store(static_cast<typename Act<AF32>::type*>(out), static_cast<size_t>(p) * n + c,
+                   g * sigmoidf_(slope * g) * (u + shift));
+}
+
 // ---------------------------------------------------------------- latent attention: the cached row
 // One wave per token: c = rms_norm(proj[t, col0 : col0 + R]) * w goes to cache [blocks, 1, BS, R] at the
 // token's slot.
@@ -560,6 +614,54 @@ __global__ __launch_bounds__(256) void qkv_prep_kernel(
     ss = wave_sum(ss);
     const float r = 1.f / sqrtf(ss / static_cast<float>(Dv) + eps);
     for (int c = lane; c < Dv; c += 64) Act<CF32>::store(vd, ((blk * G + g) * BS + off) * Dv + c, v[g * Dv + c] * r);
+  }
+}
+
+// ---------------------------------------------------------------- attention whose values are its keys
+// One block per token. qk [T, ld] fp32: q [H*D] | k [G*D], no norms and no biases. The first rot_dims
+// coordinates of each head rotate in NEIGHBOURING pairs: (x[2i], x[2i+1]) turns by position * inv_freq[i].
+// The rotated key goes to the key plane [blocks, G, BS, D]; the key as projected, BEFORE the rotation, is
+// the value and goes to the value plane of the same shape (no value plane is given when nothing rotates:
+// one plane serves as both). The angle is formed and reduced to [-pi, pi] in fp64 (frequencies fp64).
+template <bool CF32>
+__global__ __launch_bounds__(256) void rope_pairs_write_kernel(
+    const float* __restrict__ qk, int ld, const double* __restrict__ inv_freq, const int32_t* __restrict__ positions,
+    const int32_t* __restrict__ slot_mapping, void* __restrict__ kc, void* __restrict__ vc, float* __restrict__ q_out,
+    int H, int G, int D, int BS, int rot_dims) {
+  extern __shared__ float cs_dyn[];                // cos [half], sin [half] of the token's angles
+  const int t = blockIdx.x;
+  const float* row = qk + static_cast<size_t>(t) * ld;
+  const double pos = static_cast<double>(positions[t]);
+  const int half = rot_dims >> 1;
+  const int nq = H * D, nk = G * D;
+  for (int j = threadIdx.x; j < half; j += blockDim.x) {
+    constexpr double kTwoPi = 6.283185307179586476925286766559;
+    double a = pos * inv_freq[j];
+    a -= kTwoPi * rint(a / kTwoPi);
+    float s, c;
+    sincosf(static_cast<float>(a), &s, &c);
+    cs_dyn[j] = c;
+    cs_dyn[half + j] = s;
+  }
+  __syncthreads();
+  auto rotated = [&](const float* src, int idx) {
+    const int i = idx % D;
+    const float a = src[idx];
+    if (i >= rot_dims) return a;
+    const float c = cs_dyn[i >> 1], s = cs_dyn[half + (i >> 1)];
+    const float other = src[idx - i + (i ^ 1)];
+    return (i & 1) ? a * c + other * s : a * c - other * s;
+  };
+  for (int i = threadIdx.x; i < nq; i += blockDim.x) q_out[static_cast<size_t>(t) * nq + i] = rotated(row, i);
+  const int slot = slot_mapping[t];
+  if (slot < 0) return;
+  const size_t blk = slot / BS, off = slot % BS;
+  typename Act<CF32>::type* kd = static_cast<typename Act<CF32>::type*>(kc);
+  typename Act<CF32>::type* vd = static_cast<typename Act<CF32>::type*>(vc);
+  for (int i = threadIdx.x; i < nk; i += blockDim.x) {
+    const size_t at = ((blk * G + i / D) * BS + off) * D + (i % D);
+    Act<CF32>::store(kd, at, rotated(row + nq, i));
+    if (vd != nullptr) Act<CF32>::store(vd, at, row[nq + i]);
   }
 }
 
@@ -1184,6 +1286,63 @@ LC_EXPORT int lc_glu(const void* y, void* out, int act_f32, int T, int n, int ki
   const dim3 grid(static_cast<unsigned>((total + 255) / 256)), block(256);
   if (act_f32) glu_kernel<true><<<grid, block, 0, st>>>(static_cast<const float*>(y), out, total, n, kind);
   else glu_kernel<false><<<grid, block, 0, st>>>(static_cast<const float*>(y), out, total, n, kind);
+  LC_RETURN_LAST_ERROR();
+}
+
+LC_EXPORT int lc_add_dyt(void* x, const void* y, float mult, float alpha, const void* w, const void* b, void* out,
+                         int act_f32, int ldo, int T, int d, hipStream_t st) {
+  if (T <= 0) return 0;
+  if (d <= 0 || (w != nullptr && (out == nullptr || b == nullptr)) || (out != nullptr && ldo < d)) return -1;
+  if (y == nullptr && out == nullptr) return 0;
+  const long long total = static_cast<long long>(T) * d;
+  const bool v4 = d % 4 == 0 && ldo % 4 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0;
+  const long long threads = v4 ? total / 4 : total;
+  const dim3 grid(static_cast<unsigned>((threads + 255) / 256)), block(256);
+#define LC_AD(A32, V)                                                                                                  \
+  add_dyt_kernel<A32, V><<<grid, block, 0, st>>>(static_cast<float*>(x), static_cast<const float*>(y), mult, alpha,   \
+                                                 static_cast<const float*>(w), static_cast<const float*>(b), out, ldo, \
+                                                 total, d)
+  if (act_f32 && v4) LC_AD(true, 4);
+  else if (act_f32) LC_AD(true, 1);
+  else if (v4) LC_AD(false, 4);
+  else LC_AD(false, 1);
+#undef LC_AD
+  LC_RETURN_LAST_ERROR();
+}
+
+LC_EXPORT int lc_glu_clamped(const void* y, int ld, int col_gate, int col_up, int n, float limit, float slope, float shift,
+                             const void* slot_of, const void* wts, void* out, int act_f32, int rows, hipStream_t st) {
+  if (rows <= 0 || n <= 0) return 0;
+  if (col_gate < 0 || col_up < 0 || ld < col_gate + n || ld < col_up + n || (wts != nullptr && slot_of == nullptr)) return -1;
+  const long long total = static_cast<long long>(rows) * n;
+  const dim3 grid(static_cast<unsigned>((total + 255) / 256)), block(256);
+  if (act_f32)
+    glu_clamped_kernel<true><<<grid, block, 0, st>>>(static_cast<const float*>(y), ld, col_gate, col_up, n, limit, slope,
+                                                     shift, static_cast<const int32_t*>(slot_of),
+                                                     static_cast<const float*>(wts), out, total);
+  else
+    glu_clamped_kernel<false><<<grid, block, 0, st>>>(static_cast<const float*>(y), ld, col_gate, col_up, n, limit, slope,
+                                                      shift, static_cast<const int32_t*>(slot_of),
+                                                      static_cast<const float*>(wts), out, total);
+  LC_RETURN_LAST_ERROR();
+}
+
+LC_EXPORT int lc_rope_pairs_write(const void* qk, int ld, const void* inv_freq, const void* positions,
+                                  const void* slot_mapping, void* kc, void* vc, int cache_f32, void* q_out, int T, int H,
+                                  int G, int D, int BS, int rot_dims, hipStream_t st) {
+  if (T <= 0) return 0;
+  if (H <= 0 || G <= 0 || D <= 0 || BS <= 0 || rot_dims < 0 || rot_dims > D || (rot_dims & 1)) return -1;
+  if (ld < (H + G) * D || kc == nullptr || q_out == nullptr || (rot_dims > 0 && (vc == nullptr || inv_freq == nullptr)))
+    return -1;
+  const size_t lds = static_cast<size_t>(rot_dims > 0 ? rot_dims : 1) * sizeof(float);
+  if (lds > 64 * 1024) return -1;
+#define LC_RP(C32)                                                                                                \
+  rope_pairs_write_kernel<C32><<<dim3(T), dim3(256), lds, st>>>(                                                  \
+      static_cast<const float*>(qk), ld, static_cast<const double*>(inv_freq), static_cast<const int32_t*>(positions), \
+      static_cast<const int32_t*>(slot_mapping), kc, vc, static_cast<float*>(q_out), H, G, D, BS, rot_dims)
+  if (cache_f32) LC_RP(true);
+  else LC_RP(false);
+#undef LC_RP
   LC_RETURN_LAST_ERROR();
 }
 

@@ -1,4 +1,4 @@
-// Routed feed-forwards of hybrid decoder designs: a softmax router with a bias-corrected,
+// Routed feed-forwards of hybrid decoder designs: a softmax or sigmoid router with a bias-corrected,
 // group-limited top-k choice, a counting sort of the (token, choice) pairs by expert for any number
 // of experts, per-expert products of any shape and type over the sorted rows (fp32 accumulation on
 // the vector ALUs, like the shape-agnostic GEMM), and the fp32 mix of the chosen experts' outputs,
@@ -11,13 +11,14 @@ constexpr int kMaxTop = 32;
 constexpr int kMaxGroups = 64;
 
 // ---------------------------------------------------------------- routing
-// One wave per token. z [T, n] fp32 router logits (row stride ld). s = softmax(z); choice = s + correction; the n
+// One wave per token. z [T, n] fp32 router logits (row stride ld). s = softmax(z) (score_fn 0) or sigmoid(z), each
+// output on its own (score_fn 1); choice = s + correction (no correction given: s); the n
 // outputs form ``groups`` runs of n / groups neighbours, a run's score is its largest choice, the
 // ``keep`` best runs stay eligible (ties: the lower index); the ``top`` largest eligible choices are
 // taken (ties: the lower index) with weights s * scale.
 __global__ __launch_bounds__(256) void route_grouped_kernel(const float* __restrict__ z, int ld,
                                                             const float* __restrict__ corr, int T, int n, int top,
-                                                            int groups, int keep, float scale,
+                                                            int groups, int keep, float scale, int score_fn,
                                                             int32_t* __restrict__ ids, float* __restrict__ wts) {
   extern __shared__ float lds[];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -28,21 +29,26 @@ __global__ __launch_bounds__(256) void route_grouped_kernel(const float* __restr
   float* gs = ch + n;                               // group scores
   float* ok = gs + kMaxGroups;                      // 1: the group is eligible
   const float* zr = z + static_cast<size_t>(t) * ld;
-  float mx = -INFINITY;
-  for (int e = lane; e < n; e += 64) mx = fmaxf(mx, zr[e]);
-  mx = wave_max(mx);
-  float sum = 0.f;
-  for (int e = lane; e < n; e += 64) {
-    const float p = expf(zr[e] - mx);
-    sc[e] = p;
-    sum += p;
+  float inv = 1.f;
+  if (score_fn == 1) {
+    for (int e = lane; e < n; e += 64) sc[e] = sigmoidf_(zr[e]);
+  } else {
+    float mx = -INFINITY;
+    for (int e = lane; e < n; e += 64) mx = fmaxf(mx, zr[e]);
+    mx = wave_max(mx);
+    float sum = 0.f;
+    for (int e = lane; e < n; e += 64) {
+      const float p = expf(zr[e] - mx);
+      sc[e] = p;
+      sum += p;
+    }
+    sum = wave_sum(sum);
+    inv = 1.f / sum;
   }
-  sum = wave_sum(sum);
-  const float inv = 1.f / sum;
   for (int e = lane; e < n; e += 64) {
     const float s = sc[e] * inv;
     sc[e] = s;
-    ch[e] = s + corr[e];
+    ch[e] = corr != nullptr ? s + corr[e] : s;
   }
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
   __builtin_amdgcn_wave_barrier();
@@ -217,10 +223,13 @@ __global__ __launch_bounds__(256) void gemm_any_grouped_kernel(const void* __res
 
 // ---------------------------------------------------------------- mix of the chosen experts
 // out[t] = sum_k wts[t, k] * (ye[slot_of[t, k]] if ids[t, k] < E else h[t]) (+ shared[t]), fp32. One block per token.
+// No weights given: 1 (designs whose weight went into the expert's input). ``shared_gate`` (one logit per token,
+// row stride ld_gate): the shared expert's row is scaled by its sigmoid.
 template <bool HF32>
 __global__ __launch_bounds__(256) void moe_mix_kernel(const float* __restrict__ ye, const int32_t* __restrict__ slot_of,
                                                       const int32_t* __restrict__ ids, const float* __restrict__ wts,
                                                       const void* __restrict__ h, const float* __restrict__ shared,
+                                                      const float* __restrict__ shared_gate, int ld_gate,
                                                       float* __restrict__ out, int d, int top, int E) {
   __shared__ int src[kMaxTop];
   __shared__ float wk[kMaxTop];
@@ -228,12 +237,13 @@ __global__ __launch_bounds__(256) void moe_mix_kernel(const float* __restrict__ 
   if (threadIdx.x < top) {
     const int a = t * top + threadIdx.x;
     src[threadIdx.x] = ids[a] < E ? slot_of[a] : -1;
-    wk[threadIdx.x] = wts[a];
+    wk[threadIdx.x] = wts != nullptr ? wts[a] : 1.f;
   }
   __syncthreads();
+  const float sg = shared_gate != nullptr ? sigmoidf_(shared_gate[static_cast<size_t>(t) * ld_gate]) : 1.f;
   const typename Act<HF32>::type* hr = static_cast<const typename Act<HF32>::type*>(h) + static_cast<size_t>(t) * d;
   for (int c = threadIdx.x; c < d; c += blockDim.x) {
-    float acc = shared != nullptr ? shared[static_cast<size_t>(t) * d + c] : 0.f;
+    float acc = shared != nullptr ? sg * shared[static_cast<size_t>(t) * d + c] : 0.f;
     for (int k = 0; k < top; ++k)
       acc += wk[k] * (src[k] >= 0 ? ye[static_cast<size_t>(src[k]) * d + c] : Act<HF32>::load(hr, c));
     out[static_cast<size_t>(t) * d + c] = acc;
@@ -244,17 +254,18 @@ __global__ __launch_bounds__(256) void moe_mix_kernel(const float* __restrict__ 
 
 // ================================================================= launchers
 LC_EXPORT int lc_route_grouped(const void* z, int ld, const void* corr, int T, int n, int top, int groups, int keep,
-                               float scale, void* ids, void* wts, hipStream_t st) {
+                               float scale, int score_fn, void* ids, void* wts, hipStream_t st) {
   if (T <= 0) return 0;
   if (ld < n) return -1;
   if (n <= 0 || top <= 0 || top > kMaxTop || top > n || groups <= 0 || groups > kMaxGroups || n % groups || keep < 1 ||
-      keep > groups || top > keep * (n / groups))
+      keep > groups || top > keep * (n / groups) || score_fn < 0 || score_fn > 1)
     return -1;
   const size_t lds = 4 * static_cast<size_t>(2 * n + 2 * kMaxGroups) * sizeof(float);
   if (lds > 64 * 1024) return -1;
   route_grouped_kernel<<<dim3((T + 3) / 4), dim3(256), lds, st>>>(static_cast<const float*>(z), ld,
                                                                  static_cast<const float*>(corr), T, n, top, groups, keep,
-                                                                 scale, static_cast<int32_t*>(ids), static_cast<float*>(wts));
+                                                                 scale, score_fn, static_cast<int32_t*>(ids),
+                                                                 static_cast<float*>(wts));
   LC_RETURN_LAST_ERROR();
 }
 
@@ -296,17 +307,21 @@ LC_EXPORT int lc_gemm_any_grouped(const void* A, int a_f32, int lda, const void*
 }
 
 LC_EXPORT int lc_moe_mix(const void* ye, const void* slot_of, const void* ids, const void* wts, const void* h, int h_f32,
-                         const void* shared, void* out, int T, int d, int top, int E, hipStream_t st) {
+                         const void* shared, const void* shared_gate, int ld_gate, void* out, int T, int d, int top, int E,
+                         hipStream_t st) {
   if (T <= 0) return 0;
-  if (d <= 0 || top <= 0 || top > kMaxTop) return -1;
+  if (d <= 0 || top <= 0 || top > kMaxTop || (shared_gate != nullptr && (shared == nullptr || ld_gate < 1))) return -1;
   if (h_f32)
     moe_mix_kernel<true><<<dim3(T), dim3(256), 0, st>>>(static_cast<const float*>(ye), static_cast<const int32_t*>(slot_of),
                                                         static_cast<const int32_t*>(ids), static_cast<const float*>(wts), h,
-                                                        static_cast<const float*>(shared), static_cast<float*>(out), d, top, E);
+                                                        static_cast<const float*>(shared),
+                                                        static_cast<const float*>(shared_gate), ld_gate,
+                                                        static_cast<float*>(out), d, top, E);
   else
     moe_mix_kernel<false><<<dim3(T), dim3(256), 0, st>>>(static_cast<const float*>(ye), static_cast<const int32_t*>(slot_of),
                                                          static_cast<const int32_t*>(ids), static_cast<const float*>(wts), h,
-                                                         static_cast<const float*>(shared), static_cast<float*>(out), d, top,
-                                                         E);
+                                                         static_cast<const float*>(shared),
+                                                         static_cast<const float*>(shared_gate), ld_gate,
+                                                         static_cast<float*>(out), d, top, E);
   LC_RETURN_LAST_ERROR();
 }

@@ -2,9 +2,27 @@
 paged cache, latent attention over a cache of compressed rows, minGRU, gated linear attention or
 mLSTM -- around an fp32 residual stream.
 
-Two designs are served, told apart by ``architecture`` in ``config.json`` (``DESIGNS``); the file lists
+Three designs are served, told apart by ``architecture`` in ``config.json`` (``DESIGNS``); the file lists
 the layers (``layers[i].type``, ``.mixer`` sizes, ``.mlp``), and every size and constant comes from
 there or from a tensor's shape.
+
+Surevik (pre-norm, Dynamic Tanh norms):
+
+* ``x = embed[token] * embedding.scale``; a layer computes ``x += m * mixer(n1(x))`` and, if it has a
+  feed-forward, ``x += m * ff(n2(x))`` with ``m = residual_mult`` and ``n(x) = tanh(alpha x) * w + b``
+  (no mean, no variance; a scalar ``alpha``, vectors ``w``, ``b``); logits are ``embed . n_final(x)``, the
+  embedding table itself without its scale;
+* ``loop``: the layers ``start .. stop - 1`` run ``times`` times in a row with the same weights, every pass
+  over cache planes of its own; each pass begins with ``x <- W_in [x; x0]`` (``x0``: the embedding output);
+* ``attention``: ``q = W_q h``, ``k = W_k h``, no biases, no norms, and no value projection: the values
+  are the keys as projected. q and k (not the values) rotate in neighbouring coordinate pairs (2i, 2i + 1)
+  over the first ``rot.dims`` coordinates of each head; softmax over the last ``mask.size`` positions
+  (the row's own included); grouped key/value heads;
+* feed-forward: a routed mixture whose router scores are ``sigmoid(W_r h)``; the ``top`` best experts
+  are taken with their scores as weights (not renormalised), and the weight multiplies the expert's
+  INPUT; an expert is ``down(g * sigmoid(1.702 g) * (u + 1))`` with ``g = min(gate h, limit)``,
+  ``u = clamp(up h, -limit, limit)``; a shared expert of the same form runs for every token, scaled by
+  ``sigmoid(W_sg h)``.
 
 Telurax (pre-norm):
 
@@ -70,15 +88,26 @@ class Design:
     pre_norm: bool = False          # norms with a weight per coordinate on the sublayer INPUTS (else: one-gain norms on the outputs)
     norm_offset: float = 0.0        # stored norm weights are offsets from this value
     pos_base: float = 0.0           # > 0: a sinusoidal position vector of this base is added to the embedding
-    dense_ff: str = "relu2"         # dense feed-forward: down(relu(up x)^2) | "glu_relu": down(relu(gate x) * up x)
+    dense_ff: str = "relu2"         # dense feed-forward: down(relu(up x)^2) | "glu_relu": down(relu(gate x) * up x) | "": none
+    norm: str = "rms"               # "dyt": Dynamic Tanh, tanh(alpha x) * w + b (tensors <name>, <name>.b, <name>.alpha)
+    tied_head: bool = False         # logits from the embedding table (no ``head`` tensor)
+    attention: str = "normed"       # what the ``attention`` mixer is: "normed" (biases, whole-projection q / k norms,
+                                    # rotate-half pairs, unit-RMS values, ``mask.size`` = chunk) | "keys_as_values" (no
+                                    # biases or norms, values = the un-rotated keys, neighbouring pairs, ``mask.size`` = window)
+    routed_ff: str = "grouped_relu2"    # "sigmoid_clamped": sigmoid scores, weight on the expert's input, clamped gated experts
+    # constants of the clamped gated unit g * sigmoid(slope g) * (u + shift)
+    glu_slope: float = 1.702
+    glu_shift: float = 1.0
 
 
 DESIGNS: Dict[str, Design] = {
     "Nidozen": Design("Nidozen", ("attention", "mingru", "gla")),
     "Telurax": Design("Telurax", ("latent_attention", "mlstm"), pre_norm=True, norm_offset=1.0, pos_base=10000.0,
                       dense_ff="glu_relu"),
+    "Surevik": Design("Surevik", ("attention",), pre_norm=True, dense_ff="", norm="dyt", tied_head=True,
+                      attention="keys_as_values", routed_ff="sigmoid_clamped"),
 }
-MIXERS = tuple(m for d in DESIGNS.values() for m in d.mixers)
+MIXERS = tuple(dict.fromkeys(m for d in DESIGNS.values() for m in d.mixers))
 
 
 @dataclass(frozen=True)
@@ -86,7 +115,11 @@ class MoESpec:
     """A routed feed-forward: ``experts`` small relu^2 feed-forwards of width ``ff`` plus ``identity``
     experts without tensors; the router's ``experts + identity`` outputs form ``groups`` equal runs of
     neighbours of which the ``keep`` best stay eligible; ``top`` are chosen per token, weighted by their
-    softmax score times ``scale``; ``shared_ff`` > 0: a shared expert of that width runs for every token."""
+    softmax score times ``scale``; ``shared_ff`` > 0: a shared expert of that width runs for every token.
+
+    ``unit`` "clamped_glu" (with ``score`` "sigmoid"): experts are down(g * sigmoid(slope g) * (u + shift)) with
+    g = min(gate x, limit), u = clamp(up x, -limit, limit); the weight multiplies the expert's input; the
+    shared expert has a limit of its own and a sigmoid gate, one number per token."""
 
     experts: int
     ff: int
@@ -96,6 +129,14 @@ class MoESpec:
     keep: int = 1
     scale: float = 1.0
     shared_ff: int = 0
+    score: str = "softmax"
+    unit: str = "relu2"
+    limit: float = 0.0
+    shared_limit: float = 0.0
+
+    @property
+    def clamped(self) -> bool:
+        return self.unit == "clamped_glu"
 
     @property
     def outputs(self) -> int:
@@ -116,6 +157,7 @@ class LayerSpec:
     rot_dims: int = 0
     rot_base: float = 10000.0
     kv_from: int = -1            # attention: read this layer's keys and values (-1: own)
+    values_are_keys: bool = False    # attention: no norms, biases or value projection; neighbouring rotary pairs
     # gla
     tau: float = 1.0
     rank: int = 0                # width of the decay's low-rank bottleneck (from the tensor's shape)
@@ -149,6 +191,8 @@ class LayerSpec:
 
     def cache_elems(self) -> int:
         """Cached elements per token."""
+        if self.owns_kv and self.values_are_keys:     # rotated keys, and the un-rotated ones unless nothing rotates
+            return self.kv_heads * self.dim * (2 if self.rot_dims else 1)
         if self.owns_kv:
             return self.kv_heads * (self.dim + self.vdim)
         return self.kv_rank if self.type == "latent_attention" else 0
@@ -166,10 +210,28 @@ class HybridConfig:
     architecture: str = ARCHITECTURE
     embed_scale: float = 1.0
     logit_scale: float = 1.0
+    residual_mult: float = 1.0      # every sublayer output is scaled by this before it joins the stream
+    loop: Tuple[int, int, int] = (0, 0, 1)      # layers [start, stop) run ``times`` times in a row (times 1: no loop)
 
     @property
     def design(self) -> Design:
         return DESIGNS[self.architecture]
+
+    @property
+    def looped(self) -> bool:
+        return self.loop[2] != 1 or self.loop[1] > self.loop[0]
+
+    @property
+    def runs(self) -> Tuple[Tuple[int, bool], ...]:
+        """The layer runs of one forward pass in order: (layer, whether the stream is re-injected before
+        it). Run r has cache / state planes of its own: a looped layer has one set per pass."""
+        start, stop, times = self.loop
+        if not self.looped:
+            return tuple((i, False) for i in range(len(self.layers)))
+        out = [(i, False) for i in range(start)]
+        for _ in range(times):
+            out += [(i, i == start) for i in range(start, stop)]
+        return tuple(out + [(i, False) for i in range(stop, len(self.layers))])
 
     @property
     def num_layers(self) -> int:
@@ -188,13 +250,13 @@ class HybridConfig:
         return max([l.kv_heads for l in self.layers if l.type == "attention"] or [1])
 
     def kv_elems_per_token(self) -> int:
-        return sum(l.cache_elems() for l in self.layers)
+        return sum(self.layers[i].cache_elems() for i, _ in self.runs)
 
     def kv_bytes_per_token(self, bytes_per_elem: int = 2) -> int:
         return self.kv_elems_per_token() * bytes_per_elem
 
     def state_floats(self) -> int:
-        return sum(l.state_size() for l in self.layers)
+        return sum(self.layers[i].state_size() for i, _ in self.runs)
 
     def param_count(self) -> int:
         return sum(_numel(s) for s in param_shapes(self).values())
@@ -208,6 +270,12 @@ class HybridConfig:
         if self.architecture not in DESIGNS:
             raise ValueError(f"{self.name}: unknown design {self.architecture!r} (known: {', '.join(DESIGNS)})")
         known = self.design.mixers
+        start, stop, times = self.loop
+        if self.looped:
+            if not (0 <= start < stop <= len(self.layers)) or times < 1:
+                raise ValueError(f"{self.name}: loop: 0 <= start < stop <= layers and times >= 1 are needed")
+            if any(l.kv_from >= 0 for l in self.layers):
+                raise ValueError(f"{self.name}: looped layers and shared keys (kv_from) do not combine")
         if self.design.pos_base > 0 and self.hidden_size % 2:
             raise ValueError(f"{self.name}: a sinusoidal position vector needs an even width")
         for i, l in enumerate(self.layers):
@@ -221,6 +289,9 @@ class HybridConfig:
                 raise ValueError(f"{self.name}: layer {i}: mLSTM takes dim <= 256 and a gate cap >= 0")
             if l.moe is not None:
                 m = l.moe
+                if m.clamped and (m.score != "sigmoid" or m.identity or not m.limit > 0 or (m.shared_ff and not m.shared_limit > 0)):
+                    raise ValueError(f"{self.name}: layer {i}: clamped gated experts take sigmoid scores, positive limits "
+                                     f"and no identity experts")
                 if m.experts <= 0 or m.ff <= 0 or m.identity < 0 or m.top <= 0 or m.groups <= 0 or m.outputs % m.groups:
                     raise ValueError(f"{self.name}: layer {i}: experts, their width and `top` are needed, and the groups "
                                      f"must divide experts + identity")
@@ -239,6 +310,8 @@ class HybridConfig:
                     raise ValueError(f"{self.name}: layer {i}: rot.dims must be even and at most dim")
                 if l.vdim > 256:
                     raise ValueError(f"{self.name}: layer {i}: the attention kernel takes vdim <= 256")
+                if l.values_are_keys and (l.vdim != l.dim or l.kv_from >= 0 or l.chunk):
+                    raise ValueError(f"{self.name}: layer {i}: values that are the keys have the keys' width (vdim = dim)")
                 if l.kv_from >= 0:
                     src = self.layers[l.kv_from] if l.kv_from < i else None
                     if src is None or not src.owns_kv:
@@ -260,15 +333,27 @@ def _mlp_of(name: str, i: int, mlp: Optional[dict], design: Design):
     if mlp is None:
         return 0, None
     kind = mlp.get("kind", "dense")
+    if kind == "dense" and not design.dense_ff:
+        raise ValueError(f"{name}: layer {i}: {design.name} has no dense feed-forward")
     if kind == "dense":
         return int(mlp["ff"]), None
     if kind != "moe" or not design.pre_norm:
         raise ValueError(f"{name}: layer {i}: feed-forward kind {kind!r} is not supported")
     r, g = mlp["router"], mlp["router"].get("groups") or {}
     shared = mlp.get("shared") or {}
+    if design.routed_ff == "sigmoid_clamped":
+        return 0, MoESpec(experts=int(r["experts"]), ff=int(mlp["expert"]["ff"]), top=int(r["top"]),
+                          shared_ff=int(shared.get("ff", 0)), score="sigmoid", unit="clamped_glu",
+                          limit=float(mlp["expert"]["limit"]), shared_limit=float(shared.get("limit", 0.0)))
     return 0, MoESpec(experts=int(r["experts"]), ff=int(mlp["expert"]["ff"]), top=int(r["top"]),
                       identity=int(r.get("identity", 0)), groups=int(g.get("count", 1)), keep=int(g.get("keep", g.get("count", 1))),
                       scale=float(r.get("scale", 1.0)), shared_ff=int(shared.get("ff", 0)))
+
+
+def _loop_of(loop: Optional[dict]) -> Tuple[int, int, int]:
+    if not loop:
+        return (0, 0, 1)
+    return (int(loop["start"]), int(loop["stop"]), int(loop.get("times", 1)))
 
 
 def config_from_dict(c: dict, name: str = "hybrid", tensor_shapes: Optional[Dict[str, tuple]] = None) -> HybridConfig:
@@ -284,7 +369,13 @@ def config_from_dict(c: dict, name: str = "hybrid", tensor_shapes: Optional[Dict
         if t not in design.mixers:
             raise ValueError(f"{name}: layer {i}: unknown mixer {t!r} (known: {', '.join(design.mixers)})")
         ff, moe = _mlp_of(name, i, L.get("mlp"), design)
-        if t == "attention":
+        if t == "attention" and design.attention == "keys_as_values":
+            mask, rot = m.get("mask") or {}, m.get("rot") or {}
+            layers.append(LayerSpec(t, heads=int(m["heads"]), kv_heads=int(m.get("kv_heads", m["heads"])),
+                                    dim=int(m["dim"]), vdim=int(m.get("vdim", m["dim"])), scale=float(m["scale"]),
+                                    window=int(mask.get("size", 0)), rot_dims=int(rot.get("dims", 0)),
+                                    rot_base=float(rot.get("base", 10000.0)), values_are_keys=True, ff=ff, moe=moe))
+        elif t == "attention":
             mask, rot = m.get("mask") or {}, m.get("rot") or {}
             kvf = m.get("kv_from")
             layers.append(LayerSpec(t, heads=int(m["heads"]), kv_heads=int(m.get("kv_heads", m["heads"])),
@@ -311,7 +402,8 @@ def config_from_dict(c: dict, name: str = "hybrid", tensor_shapes: Optional[Dict
                        rms_eps=float(c["norm"]["eps"]), layers=tuple(layers),
                        max_position=int(c.get("max_position", 1 << 20)), model_type=arch.lower(), architecture=arch,
                        embed_scale=float((c.get("embedding") or {}).get("scale", 1.0)),
-                       logit_scale=float(c.get("logit_scale", 1.0)))
+                       logit_scale=float(c.get("logit_scale", 1.0)), residual_mult=float(c.get("residual_mult", 1.0)),
+                       loop=_loop_of(c.get("loop")))
     cfg.validate()
     return cfg
 
@@ -319,7 +411,10 @@ def config_from_dict(c: dict, name: str = "hybrid", tensor_shapes: Optional[Dict
 def config_to_dict(cfg: HybridConfig) -> dict:
     layers = []
     for l in cfg.layers:
-        if l.type == "attention":
+        if l.type == "attention" and l.values_are_keys:
+            m = {"heads": l.heads, "kv_heads": l.kv_heads, "dim": l.dim, "vdim": l.vdim, "scale": l.scale,
+                 "mask": {"size": l.window}, "rot": {"dims": l.rot_dims, "base": l.rot_base}}
+        elif l.type == "attention":
             m = {"heads": l.heads, "kv_heads": l.kv_heads, "dim": l.dim, "vdim": l.vdim, "scale": l.scale,
                  "mask": {"size": l.chunk} if not l.window else {"size": l.chunk, "window": l.window},
                  "rot": {"dims": l.rot_dims, "base": l.rot_base}}
@@ -334,7 +429,11 @@ def config_to_dict(cfg: HybridConfig) -> dict:
         else:
             m = {"heads": l.heads, "dim": l.dim, "vdim": l.vdim, "gate_cap": l.gate_cap}
         mlp = {"kind": "dense", "ff": l.ff} if l.ff else None
-        if l.moe is not None:
+        if l.moe is not None and l.moe.clamped:
+            e = l.moe
+            mlp = {"kind": "moe", "expert": {"ff": e.ff, "limit": e.limit}, "router": {"experts": e.experts, "top": e.top},
+                   "shared": {"ff": e.shared_ff, "limit": e.shared_limit} if e.shared_ff else None}
+        elif l.moe is not None:
             e = l.moe
             mlp = {"kind": "moe", "expert": {"ff": e.ff},
                    "router": {"experts": e.experts, "identity": e.identity, "top": e.top, "scale": e.scale,
@@ -345,7 +444,12 @@ def config_to_dict(cfg: HybridConfig) -> dict:
            "norm": {"eps": cfg.rms_eps}, "layers": layers}
     if cfg.design.pre_norm:
         out["embedding"] = {"scale": cfg.embed_scale}
+    if cfg.design.pre_norm and not cfg.design.tied_head:
         out["logit_scale"] = cfg.logit_scale
+    if cfg.design.norm == "dyt":
+        out["residual_mult"] = cfg.residual_mult
+    if cfg.looped:
+        out["loop"] = {"start": cfg.loop[0], "stop": cfg.loop[1], "times": cfg.loop[2]}
     return out
 
 
@@ -368,13 +472,24 @@ def param_shapes(cfg: HybridConfig) -> Dict[str, tuple]:
     d = cfg.hidden_size
     norm = (d,) if cfg.design.pre_norm else ()
     out: Dict[str, tuple] = {"embed": (cfg.vocab_size, d)}
+    dyt = cfg.design.norm == "dyt"
+
+    def norm_tensors(name: str) -> None:
+        out[name] = norm
+        if dyt:
+            out[name + ".b"], out[name + ".alpha"] = (d,), ()
+    if cfg.looped:
+        out["loop.in"] = (d, 2 * d)
     for i, l in enumerate(cfg.layers):
         p = f"l{i}."
-        out[p + "norm1"] = norm
+        norm_tensors(p + "norm1")
         if l.has_ff:
-            out[p + "norm2"] = norm
+            norm_tensors(p + "norm2")
         m = p + "mix."
-        if l.type == "attention":
+        if l.type == "attention" and l.values_are_keys:
+            out[m + "q"], out[m + "k"] = (l.heads * l.dim, d), (l.kv_heads * l.dim, d)
+            out[m + "o"] = (d, l.heads * l.vdim)
+        elif l.type == "attention":
             out[m + "q"], out[m + "q.b"], out[m + "q.norm"] = (l.heads * l.dim, d), (l.heads * l.dim,), (l.heads * l.dim,)
             if l.owns_kv:
                 out[m + "k"], out[m + "k.b"] = (l.kv_heads * l.dim, d), (l.kv_heads * l.dim,)
@@ -408,16 +523,23 @@ def param_shapes(cfg: HybridConfig) -> Dict[str, tuple]:
         if l.moe is not None:
             e = l.moe
             for j in range(e.experts):
+                if e.clamped:
+                    out[f + f"e{j}.gate"] = (e.ff, d)
                 out[f + f"e{j}.up"], out[f + f"e{j}.down"] = (e.ff, d), (d, e.ff)
-            out[f + "router"], out[f + "correction"] = (e.outputs, d), (e.outputs,)
+            out[f + "router"] = (e.outputs, d)
+            if not e.clamped:
+                out[f + "correction"] = (e.outputs,)
             if e.shared_ff:
+                if e.clamped:
+                    out[f + "shared.gate"], out[f + "shared.sg"] = (e.shared_ff, d), (1, d)
                 out[f + "shared.up"], out[f + "shared.down"] = (e.shared_ff, d), (d, e.shared_ff)
         elif l.ff:
             if cfg.design.dense_ff == "glu_relu":
                 out[f + "gate"] = (l.ff, d)
             out[f + "up"], out[f + "down"] = (l.ff, d), (d, l.ff)
-    out["final.norm"] = norm
-    out["head"] = (cfg.vocab_size, d)
+    norm_tensors("final.norm")
+    if not cfg.design.tied_head:
+        out["head"] = (cfg.vocab_size, d)
     return out
 
 
@@ -437,7 +559,8 @@ class HybridCache:
     latent-attention layers, and the fp32 state slots of the recurrent layers, in ONE pool. Key
     planes are [blocks, G, BS, dim], value planes [blocks, G, BS, vdim], latent planes
     [blocks, 1, BS, kv_rank] (keys and values at once) in the model's activation type; a state
-    plane is [slots, size] fp32."""
+    plane is [slots, size] fp32. Planes belong to layer RUNS (``HybridConfig.runs``): a layer that a
+    loop runs several times has a set per pass; without a loop run r is layer r."""
 
     def __init__(self, cfg: HybridConfig, num_blocks: int, block_size: int, num_slots: int, device,
                  dtype: torch.dtype, alloc=None):
@@ -450,10 +573,12 @@ class HybridCache:
             at = off
             off = (off + nbytes + 255) // 256 * 256
             return at
-        for i, l in enumerate(cfg.layers):
+        for i, (li, _) in enumerate(cfg.runs):
+            l = cfg.layers[li]
             if l.owns_kv:
                 plan.append(("k", i, take(num_blocks * l.kv_heads * block_size * l.dim * es)))
-                plan.append(("v", i, take(num_blocks * l.kv_heads * block_size * l.vdim * es)))
+                if not (l.values_are_keys and l.rot_dims == 0):      # (un-rotated keys that are the values: one plane)
+                    plan.append(("v", i, take(num_blocks * l.kv_heads * block_size * l.vdim * es)))
             elif l.type == "latent_attention":
                 plan.append(("c", i, take(num_blocks * block_size * l.kv_rank * es)))
             elif l.state_size():
@@ -469,10 +594,12 @@ class HybridCache:
         self._v: Dict[int, torch.Tensor] = {}
         self._s: Dict[int, torch.Tensor] = {}
         for kind, i, at in plan:
-            l = cfg.layers[i]
+            l = cfg.layers[cfg.runs[i][0]]
             if kind == "k":
                 n = num_blocks * l.kv_heads * block_size * l.dim * es
                 self._k[i] = raw[at:at + n].view(dtype).view(num_blocks, l.kv_heads, block_size, l.dim)
+                if l.values_are_keys and l.rot_dims == 0:
+                    self._v[i] = self._k[i]
             elif kind == "v":
                 n = num_blocks * l.kv_heads * block_size * l.vdim * es
                 self._v[i] = raw[at:at + n].view(dtype).view(num_blocks, l.kv_heads, block_size, l.vdim)
@@ -483,14 +610,14 @@ class HybridCache:
                 n = max(1, num_slots) * l.state_size() * 4
                 self._s[i] = raw[at:at + n].view(torch.float32).view(max(1, num_slots), l.state_size())
 
-    def k(self, layer: int) -> torch.Tensor:
-        return self._k[layer]
+    def k(self, run: int) -> torch.Tensor:
+        return self._k[run]
 
-    def v(self, layer: int) -> torch.Tensor:
-        return self._v[layer]
+    def v(self, run: int) -> torch.Tensor:
+        return self._v[run]
 
-    def state(self, layer: int) -> torch.Tensor:
-        return self._s[layer]
+    def state(self, run: int) -> torch.Tensor:
+        return self._s[run]
 
     def copy_blocks(self, src: torch.Tensor, dst: torch.Tensor) -> None:
         # sequences with a state slot are never forked (csrc/core/kv_manager.cpp), so no block is
@@ -503,17 +630,26 @@ class HybridCache:
 
 
 @dataclass
+class DyT:
+    """A Dynamic Tanh norm: tanh(alpha x) * w + b."""
+
+    alpha: float
+    w: torch.Tensor                                 # fp32 [d]
+    b: torch.Tensor                                 # fp32 [d]
+
+
+@dataclass
 class HybridLayer:
     spec: LayerSpec
-    norm1: torch.Tensor                             # fp32 [1]
+    norm1: object                                   # fp32 [1] | fp32 [d] | DyT
     proj: ops.LinearWeight                          # fused input projections of the mixer
     out: ops.LinearWeight
-    norm2: Optional[torch.Tensor] = None
+    norm2: object = None
     up: Optional[ops.LinearWeight] = None
     down: Optional[ops.LinearWeight] = None
     q_norm: Optional[torch.Tensor] = None           # fp32 [H*D]
     k_norm: Optional[torch.Tensor] = None
-    inv_freq: Optional[torch.Tensor] = None         # fp32 [rot_dims/2]
+    inv_freq: Optional[torch.Tensor] = None         # fp32 [rot_dims/2] (fp64 for neighbouring pairs)
     decay_up: Optional[ops.LinearWeight] = None     # gla: bottleneck -> decay logits
     head_norm: Optional[torch.Tensor] = None        # gla: fp32 [vdim]; mlstm: fp32 [H*vdim]
     gate_up: Optional[ops.LinearWeight] = None      # gated dense feed-forward: gate | up
@@ -522,7 +658,7 @@ class HybridLayer:
     value_up: Optional[torch.Tensor] = None         # latent attention: [H, vdim, kv_rank]
     router: Optional[ops.LinearWeight] = None       # routed feed-forward: [experts + identity, d]
     correction: Optional[torch.Tensor] = None       # fp32 [experts + identity]
-    experts_up: object = None                       # [E, ff, d] row-major, or ops.ExpertWeights (packed for the MFMA kernels)
+    experts_up: object = None                       # [E, ff, d] ([E, 2 ff, d] = gate | up of clamped gated experts) row-major, or ops.ExpertWeights (packed for the MFMA kernels)
     experts_down: object = None                     # [E, d, ff]
     shared_up: Optional[ops.LinearWeight] = None
     shared_down: Optional[ops.LinearWeight] = None
@@ -545,6 +681,7 @@ class HybridModel:
         self.embed: Optional[torch.Tensor] = None
         self.final_norm: Optional[torch.Tensor] = None
         self.lm_head: Optional[ops.LinearWeight] = None
+        self.loop_in: Optional[ops.LinearWeight] = None     # [d, 2 d]: the stream's re-injection before every pass of a loop
         self.layers: List[HybridLayer] = []
         self._rows: Dict[int, Tuple[torch.Tensor, torch.Tensor]] = {}
         self._max_len = 1
@@ -582,18 +719,29 @@ class HybridModel:
         def f32(t: torch.Tensor) -> torch.Tensor:
             return t.to(torch.float32).reshape(-1).contiguous()
 
-        def norm_w(name: str, scale: float = 1.0) -> torch.Tensor:
+        def norm_w(name: str, scale: float = 1.0):
+            if c.design.norm == "dyt":
+                return DyT(float(load(name + ".alpha").item()), (f32(load(name)) * scale).contiguous(),
+                           (f32(load(name + ".b")) * scale).contiguous())
             # stored as an offset from the design's base value; the kernels multiply by the sum
             return ((f32(load(name)) + c.design.norm_offset) * scale).contiguous()
         self.embed = load("embed").to(dt).contiguous()
         # the logits' scale rides on the final norm's weight
         self.final_norm = norm_w("final.norm", c.logit_scale) if c.design.pre_norm else f32(load("final.norm"))
-        self.lm_head = lin(load("head"))
+        # (a tied head is the embedding table once more, in the layout of the matrix products)
+        self.lm_head = lin(load("embed" if c.design.tied_head else "head"))
+        self.loop_in = lin(load("loop.in")) if c.looped else None
         self.layers = []
         for i, l in enumerate(c.layers):
             p, m = f"l{i}.", f"l{i}.mix."
             kw = {}
-            if l.type == "attention":
+            if l.type == "attention" and l.values_are_keys:
+                half = l.rot_dims // 2
+                if half:
+                    kw["inv_freq"] = torch.tensor([l.rot_base ** (-2.0 * j / l.rot_dims) for j in range(half)],
+                                                  dtype=torch.float64).to(dev)
+                proj, out = lin(torch.cat([load(m + "q"), load(m + "k")], 0), pad=True), lin(load(m + "o"))
+            elif l.type == "attention":
                 Ws, bs = [load(m + "q")], [load(m + "q.b")]
                 if l.owns_kv:
                     Ws += [load(m + "k"), load(m + "v")]
@@ -630,7 +778,23 @@ class HybridModel:
                 kw["head_norm"] = f32(load(m + "norm"))
                 out = lin(load(m + "o"))
             f = p + "mlp."
-            if l.moe is not None:
+            if l.moe is not None and l.moe.clamped:
+                e = l.moe
+                # one product for the router's logits (32-bit: fp32 accumulation of the operands) and, when there is a
+                # shared expert, its gate | up units and its gate logit: gate | up | router | sg
+                rows = [load(f + "router")]
+                if e.shared_ff:
+                    rows = [load(f + "shared.gate"), load(f + "shared.up")] + rows + [load(f + "shared.sg")]
+                    kw["shared_down"] = lin(load(f + "shared.down"))
+                kw["router"] = lin(torch.cat(rows, 0), pad=True)
+                ups = torch.stack([torch.cat([load(f + f"e{j}.gate"), load(f + f"e{j}.up")], 0) for j in range(e.experts)])
+                downs = torch.stack([load(f + f"e{j}.down") for j in range(e.experts)])
+                if dt == torch.bfloat16 and c.hidden_size % 64 == 0 and e.ff % 64 == 0:
+                    kw["experts_up"] = ops.ExpertWeights.from_dense(ups, dev)
+                    kw["experts_down"] = ops.ExpertWeights.from_dense(downs, dev)
+                else:
+                    kw["experts_up"], kw["experts_down"] = ups.to(dt).contiguous(), downs.to(dt).contiguous()
+            elif l.moe is not None:
                 e = l.moe
                 # bf16 operands with fp32 accumulation give the router's logits in 32-bit either way
                 # (and they ride behind the shared expert's up projection, one product for both, if there is one)
@@ -678,8 +842,11 @@ class HybridModel:
             gen.manual_seed((seed * 1000003 + zlib.crc32(name.encode())) & 0x7FFFFFFFFFFFFFFF)
             offset_norm = cfg.design.norm_offset != 0.0 and name.split(".")[-1] in ("norm1", "norm2") or \
                 (cfg.design.norm_offset != 0.0 and name == "final.norm")
-            if len(shape) == 2:
-                t = torch.randn(shape, generator=gen) * (1.0 if name == "embed" else shape[1] ** -0.5)
+            if name.endswith(".alpha"):
+                t = 0.6 + 0.1 * torch.randn(shape, generator=gen)
+            elif len(shape) == 2:
+                scale = cfg.hidden_size ** -0.5 if cfg.design.tied_head else 1.0     # (the table is the head too)
+                t = torch.randn(shape, generator=gen) * (scale if name == "embed" else shape[1] ** -0.5)
             elif offset_norm:
                 t = 0.1 * torch.randn(shape, generator=gen)
             elif name.endswith("norm") or name.endswith("norm1") or name.endswith("norm2"):
@@ -696,6 +863,7 @@ class HybridModel:
 
     def weight_bytes(self) -> int:
         n = self.embed.numel() * self.embed.element_size() + self.lm_head.nbytes()
+        n += self.loop_in.nbytes() if self.loop_in is not None else 0
         for L in self.layers:
             for w in (L.proj, L.out, L.up, L.down, L.decay_up, L.gate_up, L.router, L.shared_up, L.shared_down):
                 n += w.nbytes() if w is not None else 0
@@ -771,24 +939,61 @@ class HybridModel:
     def _forward_pre_norm(self, token_ids, positions, slot_mapping, meta, lay: StepLayout, cache: HybridCache,
                           taps: Optional[list]) -> torch.Tensor:
         """Layers whose sublayers read the normed stream: every residual sum and the norm that feeds
-        the next sublayer are one launch (``ops.add_rmsnorm``)."""
-        c, dt, eps = self.cfg, self.dtype, self.cfg.rms_eps
-        x, _ = ops.embed_rows(token_ids, self.embed, None, meta.token_feed, c.embed_scale, positions, self.pos_freq)
-        xa = ops.add_rmsnorm(x, None, self.layers[0].norm1, eps, dt)
-        for i, L in enumerate(self.layers):
+        the next sublayer are one launch (``_residual_norm``). The layer runs come from the
+        configuration's loop; a run that starts a pass replaces the stream by ``W_in [x; x0]``, whose input
+        the residual step in front of it writes straight into the left half of a [T, 2 d] matrix (the
+        right half holds the embedding output, written once per step)."""
+        c, dt = self.cfg, self.dtype
+        x, _ = ops.embed_rows(token_ids, self.embed, None, meta.token_feed, c.embed_scale,
+                              positions if self.pos_freq is not None else None, self.pos_freq)
+        runs, d = c.runs, c.hidden_size
+        both = None
+        if c.looped:
+            both = torch.empty(x.shape[0], 2 * d, dtype=dt, device=x.device)
+            ops.add_dyt(x, None, 1.0, 1.0, None, None, dt, out=both[:, d:])
+            if runs[0][1]:
+                ops.add_dyt(x, None, 1.0, 1.0, None, None, dt, out=both[:, :d])
+        xa = None if runs[0][1] else self._residual_norm(x, None, self.layers[runs[0][0]].norm1)
+        for r, (i, inject) in enumerate(runs):
+            L = self.layers[i]
             l = L.spec
+            if inject:
+                x = ops.linear(both, self.loop_in, out_f32=True)
+                xa = self._residual_norm(x, None, L.norm1)
             if l.type == "latent_attention":
-                y = self._latent_attention(i, L, xa, positions, slot_mapping, lay, cache)
+                y = self._latent_attention(r, L, xa, positions, slot_mapping, lay, cache)
+            elif l.type == "mlstm":
+                y = self._mlstm(r, L, xa, positions, lay, cache)
             else:
-                y = self._mlstm(i, L, xa, positions, lay, cache)
-            nxt = self.layers[i + 1].norm1 if i + 1 < len(self.layers) else None
+                y = self._attention_kv(r, L, xa, positions, slot_mapping, lay, cache)
             if l.has_ff:
-                xa = ops.add_rmsnorm(x, y, L.norm2, eps, dt)
-                y = self._routed_ff(L, xa) if l.moe is not None else self._dense_ff(L, xa)
-            xa = ops.add_rmsnorm(x, y, nxt, eps, dt)
+                xa = self._residual_norm(x, y, L.norm2)
+                if l.moe is None:
+                    y = self._dense_ff(L, xa)
+                else:
+                    y = self._clamped_ff(L, xa) if l.moe.clamped else self._routed_ff(L, xa)
+            if r + 1 == len(runs):
+                self._residual_norm(x, y, None)
+            elif runs[r + 1][1]:
+                self._residual_norm(x, y, None, out=both[:, :d])
+            else:
+                xa = self._residual_norm(x, y, self.layers[runs[r + 1][0]].norm1)
             if taps is not None:
                 taps.append(x.clone())
         return x
+
+    def _residual_norm(self, x: torch.Tensor, y: Optional[torch.Tensor], norm, out: Optional[torch.Tensor] = None):
+        """x += m * y (when y is given) and the design's norm of the new x in the activation type (when a
+        norm is given; with ``out`` and no norm: the stream itself, cast, into that column block)."""
+        c = self.cfg
+        if c.design.norm == "dyt":
+            if norm is None:
+                return ops.add_dyt(x, y, c.residual_mult, 1.0, None, None, None, out=out)
+            return ops.add_dyt(x, y, c.residual_mult, norm.alpha, norm.w, norm.b, self.dtype, out=out)
+        xa = ops.add_rmsnorm(x, y, norm, c.rms_eps, self.dtype)
+        if out is not None:                 # the start of a loop's pass: the stream itself, cast
+            ops.add_dyt(x, None, 1.0, 1.0, None, None, None, out=out)
+        return xa
 
     def _dense_ff(self, L: HybridLayer, xa: torch.Tensor) -> torch.Tensor:
         if L.gate_up is not None:
@@ -810,6 +1015,40 @@ class HybridModel:
         act = ops.grouped_linear(xa, sorted_src, offsets, L.experts_up, self.dtype, rows, relu2_epi=True)
         ye = ops.grouped_linear(act, None, offsets, L.experts_down, torch.float32, rows)
         return ops.moe_mix(ye, slot_of, ids, wts, xa, e.experts, shared)
+
+    def _clamped_ff(self, L: HybridLayer, xa: torch.Tensor) -> torch.Tensor:
+        """Routed feed-forward with sigmoid scores whose weight multiplies the expert's INPUT. The products are
+        linear up to the clamps, so the expert's gate | up product runs on the un-weighted rows and the weight
+        scales its fp32 result in the launch that clamps and gates it."""
+        e, des = L.spec.moe, self.cfg.design
+        sf = e.shared_ff
+        su = ops.linear(xa, L.router, out_f32=True)                 # (shared gate | shared up |) router logits (| shared gate logit)
+        z = su[:, 2 * sf:2 * sf + e.experts]
+        shared = gate = None
+        if sf:
+            act = ops.glu_clamped(su, 0, sf, sf, e.shared_limit, self.dtype, slope=des.glu_slope, shift=des.glu_shift)
+            shared = ops.linear(act, L.shared_down, out_f32=True)
+            gate = su[:, 2 * sf + e.experts:2 * sf + e.experts + 1]
+        ids, wts = ops.route_grouped(z, None, e.top, 1, 1, 1.0, score="sigmoid")
+        offsets, sorted_src, slot_of = ops.moe_sort(ids, e.experts)
+        rows = ids.numel()
+        gu = ops.grouped_linear(xa, sorted_src, offsets, L.experts_up, torch.float32, rows)
+        act = ops.glu_clamped(gu, 0, e.ff, e.ff, e.limit, self.dtype, slot_of=slot_of.view(-1), wts=wts.view(-1),
+                              slope=des.glu_slope, shift=des.glu_shift)
+        ye = ops.grouped_linear(act, None, offsets, L.experts_down, torch.float32, rows)
+        return ops.moe_mix(ye, slot_of, ids, None, xa, e.experts, shared, gate)
+
+    def _attention_kv(self, r: int, L: HybridLayer, xa, positions, slot_mapping, lay: StepLayout, cache: HybridCache):
+        """Attention whose values are its un-rotated keys, under a sliding window."""
+        l = L.spec
+        kc = cache.k(r)
+        vc = cache.v(r) if l.rot_dims else None
+        qk = ops.linear(xa, L.proj, out_f32=True)
+        q = ops.rope_pairs_write(qk, L.inv_freq, positions, slot_mapping, kc, vc, l.heads, l.kv_heads, l.dim, l.rot_dims)
+        a = ops.attn_masked(q, kc, cache.v(r), lay.block_tables, lay.cu_q, lay.row_seq, positions, l.heads, l.kv_heads, l.dim,
+                            l.vdim, l.scale, 0, l.window, self.dtype, n_portions=self._portions[0],
+                            portion_rows=self._portions[1], max_len=self._max_len)
+        return ops.linear(a, L.out, out_f32=True)
 
     def _latent_attention(self, i: int, L: HybridLayer, xa, positions, slot_mapping, lay: StepLayout, cache: HybridCache):
         l = L.spec
@@ -860,7 +1099,7 @@ class HybridModel:
     def logits(self, hidden_rows: torch.Tensor) -> torch.Tensor:
         """fp32 logits [R, V] of the given rows of the residual stream (final norm, then the head)."""
         if self.cfg.design.pre_norm:
-            xa = ops.add_rmsnorm(hidden_rows.contiguous(), None, self.final_norm, self.cfg.rms_eps, self.dtype)
+            xa = self._residual_norm(hidden_rows.contiguous(), None, self.final_norm)
         else:
             xa = ops.scalar_norm_add(hidden_rows, None, self.final_norm, self.cfg.rms_eps, self.dtype)
         return ops.linear(xa, self.lm_head, out_f32=True)

@@ -2,7 +2,7 @@
 
 A checkpoint names its family in ``config.json``: Hugging Face checkpoints by ``model_type``
 (llama, qwen2, mistral, mixtral -> ``TransformerModel``), hybrid decoders by ``architecture``
-(Nidozen, Telurax -> ``HybridModel``). ``resolve(path)`` returns the family entry; ``loader.load_model``
+(Nidozen, Telurax, Surevik -> ``HybridModel``). ``resolve(path)`` returns the family entry; ``loader.load_model``
 and ``loader.build_model`` go through it, so the engine, the back ends and the command-line
 tools take either kind of directory.
 """
@@ -24,7 +24,7 @@ class Family:
 
 # the designs models/hybrid.py serves (its ``DESIGNS``), named here so that finding a checkpoint's
 # family does not import the model code
-HYBRID_DESIGNS = ("Nidozen", "Telurax")
+HYBRID_DESIGNS = ("Nidozen", "Telurax", "Surevik")
 
 _FAMILIES: Dict[str, Family] = {}
 _BY_KEY: Dict[Tuple[str, str], str] = {}          # (config key, value) -> family name

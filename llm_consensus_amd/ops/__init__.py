@@ -1212,20 +1212,24 @@ def glu(y: torch.Tensor, act_dtype: torch.dtype, kind: str = "relu") -> torch.Te
     return out
 
 
-def route_grouped(z: torch.Tensor, correction: torch.Tensor, top: int, groups: int, keep: int, scale: float):
+def route_grouped(z: torch.Tensor, correction: Optional[torch.Tensor], top: int, groups: int, keep: int, scale: float,
+                  score: str = "softmax"):
     """Group-limited top-k routing over fp32 router logits z [T, n] (see ops.reference.route_grouped):
-    (ids int32 [T, top], weights fp32 [T, top])."""
+    (ids int32 [T, top], weights fp32 [T, top]). ``score``: softmax over the outputs, or sigmoid of each;
+    ``correction`` may be None."""
+    if score not in ("softmax", "sigmoid"):
+        raise ValueError(f"route_grouped: score function {score!r}: softmax or sigmoid")
     T, n = z.shape
     if groups < 1 or n % groups or not 1 <= keep <= groups or top > keep * (n // groups):
         raise ValueError("route_grouped: groups must divide the router's width and the kept groups hold `top` outputs")
     if not z.is_cuda:
-        return ref.route_grouped(z, correction, top, groups, keep, scale)
+        return ref.route_grouped(z, correction, top, groups, keep, scale, score)
     if z.stride(1) != 1 or z.dtype != torch.float32:
         raise ValueError("route_grouped: fp32 logits (a column slice of a wider matrix is taken as it is)")
     ids = torch.empty(T, top, dtype=torch.int32, device=z.device)
     wts = torch.empty(T, top, dtype=torch.float32, device=z.device)
-    _hip().call("lc_route_grouped", z.data_ptr(), max(z.stride(0), n), correction.data_ptr(), T, n, top, groups, keep,
-                float(scale), ids.data_ptr(), wts.data_ptr())
+    _hip().call("lc_route_grouped", z.data_ptr(), max(z.stride(0), n), _hip().ptr(correction), T, n, top, groups, keep,
+                float(scale), 1 if score == "sigmoid" else 0, ids.data_ptr(), wts.data_ptr())
     return ids, wts
 
 
@@ -1275,17 +1279,95 @@ def grouped_linear(x: torch.Tensor, row_index: Optional[torch.Tensor], offsets: 
     return y
 
 
-def moe_mix(ye: torch.Tensor, slot_of: torch.Tensor, ids: torch.Tensor, wts: torch.Tensor, h: torch.Tensor, E: int,
-            shared: Optional[torch.Tensor] = None) -> torch.Tensor:
+def moe_mix(ye: torch.Tensor, slot_of: torch.Tensor, ids: torch.Tensor, wts: Optional[torch.Tensor], h: torch.Tensor, E: int,
+            shared: Optional[torch.Tensor] = None, shared_gate: Optional[torch.Tensor] = None) -> torch.Tensor:
     """fp32 [T, d] = sum_k wts[t, k] * (ye[slot_of[t, k]] if ids[t, k] < E else h[t]) (+ shared[t]):
-    experts with ids >= E are identity experts, whose output is the feed-forward's input itself."""
+    experts with ids >= E are identity experts, whose output is the feed-forward's input itself.
+    Without ``wts`` every chosen expert counts once. ``shared_gate`` (fp32 logits [T, 1], may be a column
+    of a wider matrix): the shared expert's row is scaled by sigmoid(shared_gate[t])."""
     if not ye.is_cuda:
-        return ref.moe_mix(ye, slot_of, ids, wts, h, E, shared)
+        return ref.moe_mix(ye, slot_of, ids, wts, h, E, shared, shared_gate)
+    if shared_gate is not None and (shared is None or shared_gate.dtype != torch.float32 or shared_gate.shape != (ids.shape[0], 1)):
+        raise ValueError("moe_mix: the shared expert's gate is an fp32 [T, 1] column")
     T, top = ids.shape
     d = h.shape[1]
     if ye.dtype != torch.float32 or (shared is not None and shared.dtype != torch.float32):
         raise ValueError("moe_mix: fp32 expert outputs")
     out = torch.empty(T, d, dtype=torch.float32, device=h.device)
-    _hip().call("lc_moe_mix", ye.data_ptr(), slot_of.data_ptr(), ids.data_ptr(), wts.data_ptr(), h.contiguous().data_ptr(),
-                _f32flag(h.dtype), _hip().ptr(shared), out.data_ptr(), T, d, top, E)
+    _hip().call("lc_moe_mix", ye.data_ptr(), slot_of.data_ptr(), ids.data_ptr(), _hip().ptr(wts), h.contiguous().data_ptr(),
+                _f32flag(h.dtype), _hip().ptr(shared), _hip().ptr(shared_gate),
+                max(1, shared_gate.stride(0)) if shared_gate is not None else 0, out.data_ptr(), T, d, top, E)
+    return out
+
+
+# ---- Dynamic Tanh norms, attention whose values are its un-rotated keys, clamped gated experts (hybrid.hip) ----
+def add_dyt(x: torch.Tensor, y: Optional[torch.Tensor], mult: float, alpha: float, w: Optional[torch.Tensor],
+            b: Optional[torch.Tensor], act_dtype: Optional[torch.dtype], out: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+    """The residual step of a layer whose norm is a Dynamic Tanh, one launch: x (fp32 stream, in place)
+    += mult * y, and tanh(alpha * x) * w + b in ``act_dtype`` (w, b: fp32 [d]). Without ``y`` only the norm;
+    without ``w`` the stream itself in the activation type (or nothing, when ``act_dtype`` is None too).
+    ``out``: where the result goes, a [T, d] column block of a wider matrix (default: a new tensor)."""
+    T, d = x.shape
+    if x.dtype != torch.float32 or not x.is_contiguous():
+        raise ValueError("add_dyt: the residual stream is a contiguous fp32 tensor")
+    if y is not None and (y.shape != x.shape or y.dtype != torch.float32):
+        raise ValueError("add_dyt: the sublayer output must be fp32 of the stream's shape")
+    if out is None and act_dtype is not None:
+        out = torch.empty(T, d, dtype=act_dtype, device=x.device)
+    if out is not None and (out.shape != x.shape or out.stride(1) != 1):
+        raise ValueError("add_dyt: the output is a [T, d] block with unit column stride")
+    if not x.is_cuda:
+        ref.add_dyt(x, y, mult, alpha, w, b, out)
+        return out
+    if y is None and out is None:
+        return None
+    _hip().call("lc_add_dyt", x.data_ptr(), _hip().ptr(y.contiguous() if y is not None else None), float(mult), float(alpha),
+                _hip().ptr(w), _hip().ptr(b), _hip().ptr(out), _f32flag(out.dtype) if out is not None else 0,
+                max(out.stride(0), d) if out is not None else d, T, d)
+    return out
+
+
+def rope_pairs_write(qk: torch.Tensor, inv_freq: Optional[torch.Tensor], positions: torch.Tensor, slot_mapping: torch.Tensor,
+                     k_cache: torch.Tensor, v_cache: Optional[torch.Tensor], H: int, G: int, D: int, rot_dims: int) -> torch.Tensor:
+    """Attention pre-processing of a layer without norms or biases whose values are its keys: qk fp32
+    [T, >= (H + G) D] = q | k; the first ``rot_dims`` coordinates of each head rotate in neighbouring pairs
+    (2i, 2i + 1) by position * inv_freq[i] (``inv_freq`` fp64 [rot_dims / 2]); rotated keys are written to
+    ``k_cache`` [blocks, G, BS, D] and the keys as projected to ``v_cache`` (None when nothing rotates and one
+    plane is both). Returns the rotated q fp32 [T, H*D]."""
+    if rot_dims and (inv_freq is None or inv_freq.dtype != torch.float64 or inv_freq.numel() != rot_dims // 2 or v_cache is None):
+        raise ValueError("rope_pairs_write: rot_dims / 2 fp64 frequencies and a value plane are needed")
+    if k_cache.shape[1:] != (G, k_cache.shape[2], D) or (v_cache is not None and v_cache.shape != k_cache.shape):
+        raise ValueError("rope_pairs_write: cache planes do not fit the head sizes")
+    if not qk.is_cuda:
+        return ref.rope_pairs_write(qk, inv_freq, positions, slot_mapping, k_cache, v_cache, H, G, D, rot_dims)
+    T = qk.shape[0]
+    if qk.dtype != torch.float32 or qk.stride(1) != 1 or qk.shape[1] < (H + G) * D:
+        raise ValueError("rope_pairs_write: fp32 projections q | k")
+    q = torch.empty(T, H * D, dtype=torch.float32, device=qk.device)
+    _hip().call("lc_rope_pairs_write", qk.data_ptr(), qk.stride(0), _hip().ptr(inv_freq), positions.data_ptr(),
+                slot_mapping.data_ptr(), k_cache.data_ptr(), _hip().ptr(v_cache), _f32flag(k_cache.dtype), q.data_ptr(),
+                T, H, G, D, k_cache.shape[2], rot_dims)
+    return q
+
+
+def glu_clamped(y: torch.Tensor, col_gate: int, col_up: int, n: int, limit: float, act_dtype: torch.dtype,
+                slot_of: Optional[torch.Tensor] = None, wts: Optional[torch.Tensor] = None, slope: float = 1.702,
+                shift: float = 1.0) -> torch.Tensor:
+    """Clamped gated unit over column blocks of an fp32 matrix y: g = min(s * y[:, col_gate:+n], limit),
+    u = clamp(s * y[:, col_up:+n], -limit, limit), result g * sigmoid(slope * g) * (u + shift) in
+    ``act_dtype`` [rows of y, n]. With ``slot_of`` / ``wts`` (int32 / fp32, one entry per (token, choice)
+    pair) entry r names row slot_of[r] and its scale s = wts[r]: the expert-sorted rows of a routed
+    feed-forward whose weight multiplies the expert's input."""
+    R = y.shape[0]
+    rows = slot_of.numel() if slot_of is not None else R
+    if not y.is_cuda:
+        return ref.glu_clamped(y, col_gate, col_up, n, limit, slope, shift, slot_of, wts, act_dtype, rows)
+    if y.dtype != torch.float32 or y.stride(1) != 1 or max(col_gate, col_up) + n > y.shape[1]:
+        raise ValueError("glu_clamped: an fp32 matrix holding both column blocks")
+    if slot_of is not None and rows > R:
+        raise ValueError("glu_clamped: more work entries than rows")
+    out = torch.empty(R, n, dtype=act_dtype, device=y.device)
+    _hip().call("lc_glu_clamped", y.data_ptr(), y.stride(0) if R > 1 else max(y.stride(0), y.shape[1]), int(col_gate),
+                int(col_up), int(n), float(limit), float(slope), float(shift), _hip().ptr(slot_of), _hip().ptr(wts),
+                out.data_ptr(), _f32flag(act_dtype), rows)
     return out

@@ -73,11 +73,14 @@ _SIGNATURES = {
     "lc_head_linear": [_P, _I, _I, _P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _P],
     "lc_mlstm_scan": [_P, _I, _P, _L, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _P, _P, _P],
     "lc_glu": [_P, _P, _I, _I, _I, _I, _P],
+    "lc_add_dyt": [_P, _P, _F, _F, _P, _P, _P, _I, _I, _I, _I, _P],
+    "lc_glu_clamped": [_P, _I, _I, _I, _I, _F, _F, _F, _P, _P, _P, _I, _I, _P],
+    "lc_rope_pairs_write": [_P, _I, _P, _P, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _P],
     # routed feed-forwards of hybrid decoders (hybrid_moe.hip)
-    "lc_route_grouped": [_P, _I, _P, _I, _I, _I, _I, _I, _F, _P, _P, _P],
+    "lc_route_grouped": [_P, _I, _P, _I, _I, _I, _I, _I, _F, _I, _P, _P, _P],
     "lc_moe_sort": [_P, _I, _I, _I, _P, _P, _P, _P],
     "lc_gemm_any_grouped": [_P, _I, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _P],
-    "lc_moe_mix": [_P, _P, _P, _P, _P, _I, _P, _P, _I, _I, _I, _I, _P],
+    "lc_moe_mix": [_P, _P, _P, _P, _P, _I, _P, _P, _I, _P, _I, _I, _I, _I, _P],
 }
 _RESTYPES = {"lc_scan_scratch_floats": ([_I, _I, _L, _L], c_longlong)}      # helpers that return no status
 

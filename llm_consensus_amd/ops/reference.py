@@ -530,14 +530,15 @@ def glu(y: torch.Tensor, act_dtype, kind: str = "relu") -> torch.Tensor:
     return (g * u).to(act_dtype)
 
 
-def route_grouped(z: torch.Tensor, correction: torch.Tensor, top: int, groups: int, keep: int, scale: float):
-    """Router over fp32 logits z [T, n]: s = softmax(z); choice = s + correction; the n outputs form
+def route_grouped(z: torch.Tensor, correction: Optional[torch.Tensor], top: int, groups: int, keep: int, scale: float,
+                  score: str = "softmax"):
+    """Router over fp32 logits z [T, n]: s = softmax(z) (or sigmoid(z), each output on its own); choice = s + correction; the n outputs form
     ``groups`` equal runs of neighbours, a run's score is its largest choice, only the ``keep`` best runs
     stay eligible; the ``top`` largest eligible choices are taken (ties: the lower index) with weights
     s * scale. Returns (ids int32 [T, top], weights fp32 [T, top])."""
     T, n = z.shape
-    s = torch.softmax(z.float(), -1)
-    ch = s + correction.float()
+    s = torch.softmax(z.float(), -1) if score == "softmax" else torch.sigmoid(z.float())
+    ch = s + correction.float() if correction is not None else s.clone()
     if groups > 1 and keep < groups:
         gs = ch.view(T, groups, n // groups).max(-1).values
         order = torch.argsort(gs, dim=-1, descending=True, stable=True)[:, :keep]
@@ -563,12 +564,66 @@ def grouped_linear(x: torch.Tensor, row_index: Optional[torch.Tensor], offsets: 
     return y.to(out_dtype)
 
 
-def moe_mix(ye: torch.Tensor, slot_of: torch.Tensor, ids: torch.Tensor, wts: torch.Tensor, h: torch.Tensor, E: int,
-            shared: Optional[torch.Tensor]) -> torch.Tensor:
+def moe_mix(ye: torch.Tensor, slot_of: torch.Tensor, ids: torch.Tensor, wts: Optional[torch.Tensor], h: torch.Tensor, E: int,
+            shared: Optional[torch.Tensor], shared_gate: Optional[torch.Tensor] = None) -> torch.Tensor:
     """fp32 [T, d]: sum_k wts[t, k] * (ye[slot_of[t, k]] for ids < E, h[t] itself for the identity experts
-    ids >= E) + shared[t]."""
+    ids >= E) + shared[t] (times sigmoid(shared_gate[t]) when gate logits [T, 1] are given); no weights: 1."""
     T, top = ids.shape
     rows = ye[slot_of.long()].float().view(T, top, -1)
     rows = torch.where((ids >= E)[:, :, None], h.float()[:, None, :], rows)
-    out = (rows * wts.float()[:, :, None]).sum(1)
-    return out + shared.float() if shared is not None else out
+    out = (rows * wts.float()[:, :, None]).sum(1) if wts is not None else rows.sum(1)
+    if shared is None:
+        return out
+    return out + (shared.float() * torch.sigmoid(shared_gate.float().reshape(T, 1)) if shared_gate is not None else shared.float())
+
+
+def add_dyt(x: torch.Tensor, y: Optional[torch.Tensor], mult: float, alpha: float, w: Optional[torch.Tensor],
+            b: Optional[torch.Tensor], out: Optional[torch.Tensor]) -> None:
+    """x (fp32, in place) += mult * y; ``out`` (a view, any type) <- tanh(alpha x) * w + b, or x itself without w."""
+    if y is not None:
+        x.add_(y.float(), alpha=mult)
+    if out is not None:
+        out.copy_((torch.tanh(alpha * x) * w.float() + b.float()) if w is not None else x)
+
+
+def rope_pairs(x: torch.Tensor, positions: torch.Tensor, dims: int, inv_freq: torch.Tensor) -> torch.Tensor:
+    """x fp32 [T, heads, D]: in the first ``dims`` coordinates of each head the neighbours (2i, 2i + 1) turn by
+    position * inv_freq[i] (fp64 angles); the rest pass."""
+    if dims == 0:
+        return x
+    ang = positions.double()[:, None] * inv_freq.double()[None, :]
+    c, s = torch.cos(ang).float()[:, None, :], torch.sin(ang).float()[:, None, :]
+    u, v = x[..., 0:dims:2], x[..., 1:dims:2]
+    rot = torch.stack([u * c - v * s, v * c + u * s], -1).reshape(*x.shape[:-1], dims)
+    return torch.cat([rot, x[..., dims:]], -1)
+
+
+def rope_pairs_write(qk: torch.Tensor, inv_freq: Optional[torch.Tensor], positions, slot_mapping, k_cache: torch.Tensor,
+                     v_cache: Optional[torch.Tensor], H: int, G: int, D: int, rot_dims: int) -> torch.Tensor:
+    """qk fp32 [T, >= (H + G) D] = q | k. Rotated keys go to k_cache [blocks, G, BS, D], the keys as projected
+    (before the rotation) to v_cache, the layer's values. Returns the rotated q fp32 [T, H*D]."""
+    T = qk.shape[0]
+    q = rope_pairs(qk[:, :H * D].float().view(T, H, D), positions, rot_dims, inv_freq).reshape(T, H * D)
+    k = qk[:, H * D:(H + G) * D].float().view(T, G, D)
+    BS = k_cache.shape[2]
+    slots = slot_mapping.long()
+    ok = slots >= 0
+    blk, off = slots[ok] // BS, slots[ok] % BS
+    k_cache[blk, :, off, :] = rope_pairs(k, positions, rot_dims, inv_freq)[ok].to(k_cache.dtype)
+    if v_cache is not None:
+        v_cache[blk, :, off, :] = k[ok].to(v_cache.dtype)
+    return q.contiguous()
+
+
+def glu_clamped(y: torch.Tensor, col_gate: int, col_up: int, n: int, limit: float, slope: float, shift: float,
+                slot_of: Optional[torch.Tensor], wts: Optional[torch.Tensor], act_dtype, rows: int) -> torch.Tensor:
+    """g = min(s gate, limit), u = clamp(s up, -limit, limit) -> g sigmoid(slope g) (u + shift); with a work list,
+    entry r is row slot_of[r] scaled by s = wts[r] (rows no entry names stay zero)."""
+    g, u = y[:, col_gate:col_gate + n].float(), y[:, col_up:col_up + n].float()
+    if slot_of is None:
+        s = 1.0
+    else:
+        s = torch.zeros(y.shape[0], 1, dtype=torch.float32, device=y.device)
+        s[slot_of.long().reshape(-1)[:rows], 0] = wts.float().reshape(-1)[:rows] if wts is not None else 1.0
+    g, u = torch.clamp(g * s, max=limit), torch.clamp(u * s, -limit, limit)
+    return (g * torch.sigmoid(slope * g) * (u + shift)).to(act_dtype)

@@ -347,3 +347,101 @@ def test_sorted_expert_products_on_the_packed_mfma_kernels(T, top, E, d, ff):
     real = int(off.cpu()[E])
     torch.testing.assert_close(act.float().cpu()[:real], act_ref.float()[:real], atol=3e-2, rtol=3e-2)
     torch.testing.assert_close(ye.cpu()[:real], ye_ref[:real], atol=3e-2, rtol=3e-2)
+
+
+# ---- Dynamic Tanh residual step, neighbouring rotary pairs with keys as values, clamped gated units ----
+@pytest.mark.parametrize("dt", ACTS)
+@pytest.mark.parametrize("T,d", [(3, 10), (600, 132), (1, 64)])
+def test_dynamic_tanh_residual_step(dt, T, d):
+    g = torch.Generator().manual_seed(T + d)
+    x0, y = torch.randn(T, d, generator=g), torch.randn(T, d, generator=g)
+    w, b = torch.randn(d, generator=g), torch.randn(d, generator=g)
+    x = x0.clone().to(DEV)
+    xa = ops.add_dyt(x, y.to(DEV), 0.7, 0.4, w.to(DEV), b.to(DEV), dt)
+    xr = x0.clone()
+    want = torch.empty(T, d, dtype=dt)
+    ref.add_dyt(xr, y, 0.7, 0.4, w, b, want)
+    torch.testing.assert_close(x.cpu(), xr, atol=1e-6, rtol=1e-6)
+    torch.testing.assert_close(xa.float().cpu(), want.float(), **_tol(dt))
+    # the norm alone leaves the stream as it is; the sum alone returns nothing
+    x2 = x0.clone().to(DEV)
+    torch.testing.assert_close(ops.add_dyt(x2, None, 0.7, 0.4, w.to(DEV), b.to(DEV), dt).float().cpu(),
+                               (torch.tanh(0.4 * x0) * w + b).to(dt).float(), **_tol(dt))
+    torch.testing.assert_close(x2.cpu(), x0)
+    assert ops.add_dyt(x2, y.to(DEV), 2.0, 1.0, None, None, None) is None
+    torch.testing.assert_close(x2.cpu(), x0 + 2.0 * y)
+    # the stream itself, cast, into the left and the right half of a wider matrix
+    both = torch.zeros(T, 2 * d, dtype=dt, device=DEV)
+    ops.add_dyt(x2, None, 1.0, 1.0, None, None, dt, out=both[:, d:])
+    ops.add_dyt(x2, y.to(DEV), -2.0, 1.0, None, None, dt, out=both[:, :d])
+    torch.testing.assert_close(both.float().cpu(), torch.cat([x0, x0 + 2.0 * y], 1).to(dt).float(), **_tol(dt))
+
+
+@pytest.mark.parametrize("dt", ACTS)
+@pytest.mark.parametrize("H,G,D,rot,window", [(4, 2, 32, 8, 7), (3, 3, 48, 48, 40), (2, 1, 16, 0, 5), (5, 1, 7, 6, 3), (6, 2, 64, 32, 100)])
+def test_rotary_pairs_keys_as_values_and_window_attention(dt, H, G, D, rot, window):
+    g = torch.Generator().manual_seed(H * 100 + D)
+    lens, starts = [37, 70, 1, 1], [0, 130, 55, 3]          # two portions (one continuing at place 130), two decoded tokens
+    BSZ, MB = 16, 14
+    cu, pos, rs = _seqs(lens, starts)
+    T = int(cu[-1])
+    tables = torch.randperm(4 * MB, generator=g).to(torch.int32).view(4, MB)
+    slots = torch.tensor([int(tables[b, p // BSZ]) * BSZ + p % BSZ for b, p in zip(rs.tolist(), pos.tolist())], dtype=torch.int32)
+    qk = torch.randn(T, (H + G) * D + 5, generator=g)
+    base = (torch.randn(4 * MB, G, BSZ, D, generator=g) * 0.5).to(dt)        # what earlier steps left in the pages
+    inv = torch.tensor([1e4 ** (-2.0 * j / rot) for j in range(rot // 2)], dtype=torch.float64) if rot else None
+    kc, vc = base.clone(), (base.clone() * 0.7 if rot else None)
+    kd, vd = kc.clone().to(DEV), (vc.clone().to(DEV) if rot else None)
+    q = ops.rope_pairs_write(qk.to(DEV), inv.to(DEV) if rot else None, pos.to(DEV), slots.to(DEV), kd, vd, H, G, D, rot)
+    qr = ref.rope_pairs_write(qk, inv, pos, slots, kc, vc, H, G, D, rot)
+    torch.testing.assert_close(q.cpu(), qr, atol=2e-5, rtol=2e-5)
+    torch.testing.assert_close(kd.float().cpu(), kc.float(), **_tol(dt))
+    if rot:
+        torch.testing.assert_close(vd.float().cpu(), vc.float(), **_tol(dt))
+    vv, vvd = (vc, vd) if rot else (kc, kd)
+    want = ref.attn_masked(qr, kc, vv, tables, cu, pos, H, G, D, D, 0.2, 0, window, dt)
+    for portions, rows in ((0, 0), (2, 107)):               # the row kernel for everything; matrix-core tiles for the portions
+        got = ops.attn_masked(q, kd, vvd, tables.to(DEV), cu.to(DEV), rs.to(DEV), pos.to(DEV), H, G, D, D, 0.2, 0, window, dt,
+                              n_portions=portions, portion_rows=rows, max_len=70)
+        torch.testing.assert_close(got.float().cpu(), want.float(), **_tol(dt))
+
+
+@pytest.mark.parametrize("dt", ACTS)
+def test_clamped_gated_unit(dt):
+    g = torch.Generator().manual_seed(5)
+    y = torch.randn(33, 50, generator=g) * 2
+    got = ops.glu_clamped(y.to(DEV), 3, 20, 17, 0.8, dt)
+    gate, up = y[:, 3:20].clamp(max=0.8), y[:, 20:37].clamp(-0.8, 0.8)
+    torch.testing.assert_close(got.float().cpu(), (gate * torch.sigmoid(1.702 * gate) * (up + 1)).to(dt).float(), **_tol(dt))
+    # a work list: entry r names row slot_of[r], scaled by wts[r] BEFORE the clamps
+    slot_of = torch.randperm(33, generator=g).to(torch.int32)
+    wts = torch.rand(33, generator=g)
+    got = ops.glu_clamped(y.to(DEV), 0, 25, 25, 1.5, dt, slot_of=slot_of.to(DEV), wts=wts.to(DEV), slope=1.1, shift=0.5)
+    s = torch.empty(33)
+    s[slot_of.long()] = wts
+    gate, up = (y[:, :25] * s[:, None]).clamp(max=1.5), (y[:, 25:] * s[:, None]).clamp(-1.5, 1.5)
+    torch.testing.assert_close(got.float().cpu(), (gate * torch.sigmoid(1.1 * gate) * (up + 0.5)).to(dt).float(), **_tol(dt))
+    torch.testing.assert_close(ref.glu_clamped(y, 0, 25, 25, 1.5, 1.1, 0.5, slot_of, wts, dt, 33).float(), got.float().cpu(), **_tol(dt))
+
+
+@pytest.mark.parametrize("n,top", [(6, 2), (70, 5), (3, 3), (130, 1)])
+def test_route_by_sigmoid_scores(n, top):
+    g = torch.Generator().manual_seed(n)
+    z = torch.randn(50, n + 3, generator=g)[:, 1:n + 1]           # a column slice of a wider matrix
+    ids, wts = ops.route_grouped(z.to(DEV), None, top, 1, 1, 1.0, score="sigmoid")
+    ri, rw = ref.route_grouped(z, None, top, 1, 1, 1.0, "sigmoid")
+    assert (ids.cpu() == ri).all()
+    torch.testing.assert_close(wts.cpu(), rw, atol=1e-6, rtol=1e-5)
+    torch.testing.assert_close(rw, torch.sigmoid(z).gather(1, ri.long()))
+
+
+def test_expert_mix_without_weights_under_a_gated_shared_expert():
+    g = torch.Generator().manual_seed(2)
+    T, top, E, d = 40, 3, 7, 24
+    ids = torch.stack([torch.randperm(E, generator=g)[:top] for _ in range(T)]).to(torch.int32)
+    offsets, src, slot_of = ops.moe_sort(ids.to(DEV), E)
+    ye, shared, h = torch.randn(T * top, d, generator=g), torch.randn(T, d, generator=g), torch.randn(T, d, generator=g)
+    wide = torch.randn(T, 9, generator=g)
+    got = ops.moe_mix(ye.to(DEV), slot_of, ids.to(DEV), None, h.to(DEV), E, shared.to(DEV), wide.to(DEV)[:, 4:5])
+    want = ye[slot_of.cpu().long()].view(T, top, d).sum(1) + torch.sigmoid(wide[:, 4:5]) * shared
+    torch.testing.assert_close(got.cpu(), want, atol=1e-5, rtol=1e-5)

@@ -136,7 +136,7 @@ __global__ __launch_bounds__(256) void gemm_grouped_kernel(const bf16_t* __restr
                                                            const int32_t* __restrict__ row_index,
                                                            const int32_t* __restrict__ offsets, int E,
                                                            void* __restrict__ Y, int N, int K, int ldy,
-                                                           int tiles_n) {
+                                                           int tiles_n, GluClamp glu) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -195,7 +195,10 @@ __global__ __launch_bounds__(256) void gemm_grouped_kernel(const bf16_t* __restr
   for (int i = 0; i < 4; ++i)
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      if constexpr (EPI == EPI_SWIGLU) {
+      if constexpr (EPI == EPI_GLU_CLAMPED) {
+        if (i & 1) continue;
+        store_tile_glu_clamped(acc[i][j], acc[i + 1][j], Y, glu, mbase + j * 16, nbase + i * 16, m_hi, N, ldy, lane);
+      } else if constexpr (EPI == EPI_SWIGLU) {
         if (i & 1) continue;
         store_tile<EPI>(acc[i][j], &acc[i + 1][j], Y, nullptr, mbase + j * 16, nbase + i * 16, m_hi, N, ldy, lane, 0);
       } else {
@@ -284,9 +287,9 @@ LC_EXPORT int lc_splitk_reduce(const void* part, const void* bias, void* Y, int 
 // Grouped GEMM over E experts. offsets (device, int32 [E+1]) delimit each expert's rows
 // in the expert-sorted order; total_rows bounds the launch (tiles beyond the used ones
 // exit immediately). Output rows are in sorted order.
-LC_EXPORT int lc_gemm_grouped(const void* Wp_all, long long expert_stride, const void* X,
-                              const void* row_index, const void* offsets, int E, void* Y, int total_rows,
-                              int N, int K, int n_pad, int ldy, int epi, hipStream_t stream) {
+static int launch_gemm_grouped(const void* Wp_all, long long expert_stride, const void* X, const void* row_index,
+                               const void* offsets, int E, void* Y, int total_rows, int N, int K, int n_pad, int ldy,
+                               int epi, GluClamp glu, hipStream_t stream) {
   if (total_rows <= 0) return 0;
   if (K % 64 || n_pad % 128 || N > n_pad || E < 1) return -1;
   const int tiles_n = n_pad / GT_BN;
@@ -297,15 +300,32 @@ LC_EXPORT int lc_gemm_grouped(const void* Wp_all, long long expert_stride, const
   auto x = static_cast<const bf16_t*>(X);
   auto ri = static_cast<const int32_t*>(row_index);
   auto off = static_cast<const int32_t*>(offsets);
-  if (epi == EPI_BF16)
-    gemm_grouped_kernel<EPI_BF16><<<grid, block, lds, stream>>>(w, expert_stride, x, ri, off, E, Y, N, K, ldy, tiles_n);
-  else if (epi == EPI_SWIGLU)
-    gemm_grouped_kernel<EPI_SWIGLU><<<grid, block, lds, stream>>>(w, expert_stride, x, ri, off, E, Y, N, K, ldy, tiles_n);
-  else if (epi == EPI_RELU2)
-    gemm_grouped_kernel<EPI_RELU2><<<grid, block, lds, stream>>>(w, expert_stride, x, ri, off, E, Y, N, K, ldy, tiles_n);
-  else if (epi == EPI_F32)
-    gemm_grouped_kernel<EPI_F32><<<grid, block, lds, stream>>>(w, expert_stride, x, ri, off, E, Y, N, K, ldy, tiles_n);
-  else
-    return -2;
+#define LC_GG(EPI_) \
+  gemm_grouped_kernel<EPI_><<<grid, block, lds, stream>>>(w, expert_stride, x, ri, off, E, Y, N, K, ldy, tiles_n, glu)
+  if (epi == EPI_BF16) LC_GG(EPI_BF16);
+  else if (epi == EPI_SWIGLU) LC_GG(EPI_SWIGLU);
+  else if (epi == EPI_RELU2) LC_GG(EPI_RELU2);
+  else if (epi == EPI_F32) LC_GG(EPI_F32);
+  else if (epi == EPI_GLU_CLAMPED) LC_GG(EPI_GLU_CLAMPED);
+  else return -2;
+#undef LC_GG
   LC_RETURN_LAST_ERROR();
+}
+
+LC_EXPORT int lc_gemm_grouped(const void* Wp_all, long long expert_stride, const void* X,
+                              const void* row_index, const void* offsets, int E, void* Y, int total_rows,
+                              int N, int K, int n_pad, int ldy, int epi, hipStream_t stream) {
+  if (epi == EPI_GLU_CLAMPED) return -2;
+  return launch_gemm_grouped(Wp_all, expert_stride, X, row_index, offsets, E, Y, total_rows, N, K, n_pad, ldy, epi,
+                             GluClamp{nullptr, 0.f, 0.f, 0.f}, stream);
+}
+
+// The gate | up product of clamped gated experts (n-tiles alternate gate / up): Y bf16 [rows, N / 2] is the gated
+// unit of the product scaled by row_scale[sorted position] (fp32, may be null).
+LC_EXPORT int lc_gemm_grouped_glu(const void* Wp_all, long long expert_stride, const void* X, const void* row_index,
+                                  const void* offsets, int E, void* Y, int total_rows, int N, int K, int n_pad, int ldy,
+                                  const void* row_scale, float limit, float slope, float shift, hipStream_t stream) {
+  if (N % 32) return -1;
+  return launch_gemm_grouped(Wp_all, expert_stride, X, row_index, offsets, E, Y, total_rows, N, K, n_pad, ldy,
+                             EPI_GLU_CLAMPED, GluClamp{static_cast<const float*>(row_scale), limit, slope, shift}, stream);
 }

@@ -10,9 +10,39 @@ enum Epilogue : int {
   EPI_F32 = 1,     // Y f32  [M, ldy]  (+bias); with split-K: slab blockIdx.y of [S, M, ldy], no bias
   EPI_SWIGLU = 2,  // n-tiles alternate gate/up; Y bf16 [M, N/2] = silu(gate)*up (+bias before act)
   EPI_RELU2 = 3,   // Y bf16 [M, ldy] = relu(. + bias)^2 (the grouped kernels)
+  EPI_GLU_CLAMPED = 4,  // n-tiles alternate gate/up; Y bf16 [M, N/2] = clamped gated unit with a scale per row (the grouped kernels)
+};
+
+// Constants of the clamped gated unit: with s = row_scale[row] (1 without the array), g = min(s * gate, limit),
+// u = clamp(s * up, -limit, limit), the output is g * sigmoid(slope * g) * (u + shift).
+struct GluClamp {
+  const float* row_scale;
+  float limit, slope, shift;
 };
 
 LC_DEVICE float silu(float x) { return x / (1.f + __expf(-x)); }
+
+// The clamped gated unit over a gate tile and the up tile next to it (same layout as the SwiGLU store below).
+// ``row_scale`` is indexed like the output rows.
+LC_DEVICE void store_tile_glu_clamped(const f32x4& acc, const f32x4& acc_up, void* __restrict__ Y, const GluClamp& glu,
+                                      int m0, int n0, int M, int N, int ldy, int lane) {
+  const int m = m0 + (lane & 15);
+  const int nb = n0 + 4 * (lane >> 4);
+  if (m >= M || nb >= N) return;
+  const int ob = (n0 >> 1) + 4 * (lane >> 4);
+  const float s = glu.row_scale != nullptr ? glu.row_scale[m] : 1.f;
+  float v[4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const float g = fminf(acc[r] * s, glu.limit);
+    const float u = fminf(fmaxf(acc_up[r] * s, -glu.limit), glu.limit);
+    v[r] = g / (1.f + expf(-glu.slope * g)) * (u + glu.shift);
+  }
+  u32x2 o;
+  o[0] = pack_bf16x2(v[0], v[1]);
+  o[1] = pack_bf16x2(v[2], v[3]);
+  *reinterpret_cast<u32x2*>(static_cast<bf16_t*>(Y) + static_cast<size_t>(m) * ldy + ob) = o;
+}
 
 // Stores one 16(n) x 16(m) accumulator tile. `n0`/`m0` are the tile origin.
 template <int EPI>

@@ -463,7 +463,8 @@ __global__ __launch_bounds__(512) void gemm_panel_grouped_kernel(const bf16_t* _
                                                                  const bf16_t* __restrict__ X,
                                                                  const int32_t* __restrict__ row_index,
                                                                  const int32_t* __restrict__ offsets,
-                                                                 void* __restrict__ Y, int N, int K, int ldy) {
+                                                                 void* __restrict__ Y, int N, int K, int ldy,
+                                                                 GluClamp glu) {
   using S = PanelShape<BM, true>;
   static_assert(S::P * S::DEPTH <= 63, "vmcnt is a 6-bit counter");
   extern __shared__ __attribute__((aligned(16))) char smem[];
@@ -553,7 +554,13 @@ __global__ __launch_bounds__(512) void gemm_panel_grouped_kernel(const bf16_t* _
   for (int i = 0; i < S::NT_W; ++i)
 #pragma unroll
     for (int j = 0; j < S::MT_W; ++j) {
-      if constexpr (EPI == EPI_SWIGLU) {
+      if constexpr (EPI == EPI_GLU_CLAMPED) {
+        if (i & 1) continue;
+        GluClamp mine = glu;                         // (the scale is indexed by sorted position: this expert's rows start at r0)
+        if (mine.row_scale != nullptr) mine.row_scale += r0;
+        store_tile_glu_clamped(acc[i][j], acc[(i + 1) % S::NT_W][j], Ye, mine, mbase + j * 16, nbase + i * 16, M, N, ldy,
+                               lane);
+      } else if constexpr (EPI == EPI_SWIGLU) {
         if (i & 1) continue;
         store_tile<EPI>(acc[i][j], &acc[(i + 1) % S::NT_W][j], Ye, nullptr, mbase + j * 16, nbase + i * 16, M, N, ldy,
                         lane, 0);
@@ -566,7 +573,7 @@ __global__ __launch_bounds__(512) void gemm_panel_grouped_kernel(const bf16_t* _
 template <int BM>
 int launch_panel_grouped(int epi, const bf16_t* w, long long stride, const bf16_t* x, const int32_t* ri,
                          const int32_t* off, int E, int total_rows, void* Y, int N, int K, int n_pad, int ldy,
-                         hipStream_t stream) {
+                         GluClamp glu, hipStream_t stream) {
   using S = PanelShape<BM, true>;
   const dim3 grid(n_pad / GP_BN, (total_rows + BM - 1) / BM, E), block(512);
   const int lds = S::NSTAGE * S::STAGE;
@@ -580,15 +587,19 @@ int launch_panel_grouped(int epi, const bf16_t* w, long long stride, const bf16_
                         hipFuncAttributeMaxDynamicSharedMemorySize, lds);
     (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_panel_grouped_kernel<BM, EPI_F32>),
                         hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_panel_grouped_kernel<BM, EPI_GLU_CLAMPED>),
+                        hipFuncAttributeMaxDynamicSharedMemorySize, lds);
   });
   if (epi == EPI_BF16)
-    gemm_panel_grouped_kernel<BM, EPI_BF16><<<grid, block, lds, stream>>>(w, stride, x, ri, off, Y, N, K, ldy);
+    gemm_panel_grouped_kernel<BM, EPI_BF16><<<grid, block, lds, stream>>>(w, stride, x, ri, off, Y, N, K, ldy, glu);
   else if (epi == EPI_SWIGLU)
-    gemm_panel_grouped_kernel<BM, EPI_SWIGLU><<<grid, block, lds, stream>>>(w, stride, x, ri, off, Y, N, K, ldy);
+    gemm_panel_grouped_kernel<BM, EPI_SWIGLU><<<grid, block, lds, stream>>>(w, stride, x, ri, off, Y, N, K, ldy, glu);
   else if (epi == EPI_RELU2)
-    gemm_panel_grouped_kernel<BM, EPI_RELU2><<<grid, block, lds, stream>>>(w, stride, x, ri, off, Y, N, K, ldy);
+    gemm_panel_grouped_kernel<BM, EPI_RELU2><<<grid, block, lds, stream>>>(w, stride, x, ri, off, Y, N, K, ldy, glu);
   else if (epi == EPI_F32)
-    gemm_panel_grouped_kernel<BM, EPI_F32><<<grid, block, lds, stream>>>(w, stride, x, ri, off, Y, N, K, ldy);
+    gemm_panel_grouped_kernel<BM, EPI_F32><<<grid, block, lds, stream>>>(w, stride, x, ri, off, Y, N, K, ldy, glu);
+  else if (epi == EPI_GLU_CLAMPED)
+    gemm_panel_grouped_kernel<BM, EPI_GLU_CLAMPED><<<grid, block, lds, stream>>>(w, stride, x, ri, off, Y, N, K, ldy, glu);
   else
     return -2;
   return static_cast<int>(hipGetLastError());
@@ -630,9 +641,9 @@ LC_EXPORT int lc_gemm_panel(const void* Wp, const void* X, void* Y, const void* 
 
 // Grouped skinny GEMM over E experts (see gemm_panel_grouped_kernel). total_rows <= 256 bounds the
 // rows any single expert can receive. Same row/offset conventions as lc_gemm_grouped.
-LC_EXPORT int lc_gemm_panel_grouped(const void* Wp_all, long long expert_stride, const void* X,
-                                    const void* row_index, const void* offsets, int E, void* Y, int total_rows,
-                                    int N, int K, int n_pad, int ldy, int epi, hipStream_t stream) {
+static int panel_grouped(const void* Wp_all, long long expert_stride, const void* X, const void* row_index,
+                         const void* offsets, int E, void* Y, int total_rows, int N, int K, int n_pad, int ldy, int epi,
+                         GluClamp glu, hipStream_t stream) {
   if (total_rows <= 0) return 0;
   if (K % 64 || n_pad % GP_BN || N > n_pad || E < 1) return -1;
   auto w = static_cast<const bf16_t*>(Wp_all);
@@ -642,10 +653,28 @@ LC_EXPORT int lc_gemm_panel_grouped(const void* Wp_all, long long expert_stride,
   // Panel height: about twice the mean rows per expert (the routing of a batch is never even).
   const int want = std::min(total_rows, std::max(32, 2 * ((total_rows + E - 1) / E)));
 #define LC_PG(BM_) \
-  return launch_panel_grouped<BM_>(epi, w, expert_stride, x, ri, off, E, total_rows, Y, N, K, n_pad, ldy, stream)
+  return launch_panel_grouped<BM_>(epi, w, expert_stride, x, ri, off, E, total_rows, Y, N, K, n_pad, ldy, glu, stream)
   if (want <= 32) LC_PG(32);
   if (want <= 64) LC_PG(64);
   if (want <= 128) LC_PG(128);
   LC_PG(256);
 #undef LC_PG
+}
+
+LC_EXPORT int lc_gemm_panel_grouped(const void* Wp_all, long long expert_stride, const void* X,
+                                    const void* row_index, const void* offsets, int E, void* Y, int total_rows,
+                                    int N, int K, int n_pad, int ldy, int epi, hipStream_t stream) {
+  if (epi == EPI_GLU_CLAMPED) return -2;
+  return panel_grouped(Wp_all, expert_stride, X, row_index, offsets, E, Y, total_rows, N, K, n_pad, ldy, epi,
+                       GluClamp{nullptr, 0.f, 0.f, 0.f}, stream);
+}
+
+// The gate | up product of clamped gated experts over one panel per expert (see lc_gemm_grouped_glu).
+LC_EXPORT int lc_gemm_panel_grouped_glu(const void* Wp_all, long long expert_stride, const void* X, const void* row_index,
+                                        const void* offsets, int E, void* Y, int total_rows, int N, int K, int n_pad,
+                                        int ldy, const void* row_scale, float limit, float slope, float shift,
+                                        hipStream_t stream) {
+  if (N % 32) return -1;
+  return panel_grouped(Wp_all, expert_stride, X, row_index, offsets, E, Y, total_rows, N, K, n_pad, ldy, EPI_GLU_CLAMPED,
+                       GluClamp{static_cast<const float*>(row_scale), limit, slope, shift}, stream);
 }

@@ -111,12 +111,14 @@ __global__ __launch_bounds__(256) void route_grouped_kernel(const float* __restr
 
 // ---------------------------------------------------------------- sort of the pairs by expert
 // One block. ids [A] (A = T * top, pair a = token a / top). offsets [n + 1]: first sorted position of
-// every expert; sorted_src [A]: token of every sorted position; slot_of [A]: sorted position of pair a.
+// every expert; sorted_src [A]: token of every sorted position; slot_of [A]: sorted position of pair a;
+// with ``wts`` [A] also sorted_wts [A]: the pair's weight at its sorted position.
 // The order inside an expert is whatever the atomics give; every row is computed on its own, so
 // the values do not depend on it.
 __global__ __launch_bounds__(1024) void moe_sort_kernel(const int32_t* __restrict__ ids, int A, int top, int n,
                                                         int32_t* __restrict__ offsets, int32_t* __restrict__ sorted_src,
-                                                        int32_t* __restrict__ slot_of) {
+                                                        int32_t* __restrict__ slot_of, const float* __restrict__ wts,
+                                                        float* __restrict__ sorted_wts) {
   extern __shared__ int cnt[];                      // [n] counts, then [n] cursors
   int* cur = cnt + n;
   for (int e = threadIdx.x; e < n; e += blockDim.x) cnt[e] = 0;
@@ -145,6 +147,7 @@ __global__ __launch_bounds__(1024) void moe_sort_kernel(const int32_t* __restric
     const int p = atomicAdd(&cur[e], 1);
     sorted_src[p] = a / top;
     slot_of[a] = p;
+    if (wts != nullptr) sorted_wts[p] = wts[a];
   }
 }
 
@@ -270,12 +273,12 @@ LC_EXPORT int lc_route_grouped(const void* z, int ld, const void* corr, int T, i
 }
 
 LC_EXPORT int lc_moe_sort(const void* ids, int T, int top, int n, void* offsets, void* sorted_src, void* slot_of,
-                          hipStream_t st) {
+                          const void* wts, void* sorted_wts, hipStream_t st) {
   if (T <= 0) return 0;
-  if (top <= 0 || n <= 0 || n > 4096) return -1;
+  if (top <= 0 || n <= 0 || n > 4096 || (wts != nullptr && sorted_wts == nullptr)) return -1;
   moe_sort_kernel<<<dim3(1), dim3(1024), 2 * static_cast<size_t>(n) * sizeof(int), st>>>(
       static_cast<const int32_t*>(ids), T * top, top, n, static_cast<int32_t*>(offsets), static_cast<int32_t*>(sorted_src),
-      static_cast<int32_t*>(slot_of));
+      static_cast<int32_t*>(slot_of), static_cast<const float*>(wts), static_cast<float*>(sorted_wts));
   LC_RETURN_LAST_ERROR();
 }
 

@@ -1,6 +1,6 @@
-"""Prefill and decode throughput of the hybrid decoders (Nidozen, Telurax) beside each other and a
+"""Prefill and decode throughput of the hybrid decoders (Nidozen, Telurax, Surevik) beside each other and a
 Llama-shaped transformer of equal width, depth and head sizes (``bench.py --hybrid``,
-``--hybrid-models telurax,nidozen,llama``). Random weights, synthetic tokens.
+``--hybrid-models surevik,telurax,nidozen,llama``). Random weights, synthetic tokens.
 
 Per size: one prompt of ``prompt`` tokens goes through each engine as a single step (prefill
 tokens/s), then ``batch`` requests decode ``new`` tokens each from recorded steps (decode tokens/s).
@@ -8,7 +8,10 @@ The hybrid stack repeats (attention, minGRU, attention on the first layer's keys
 linear attention); the Telurax stack alternates mLSTM layers with a gated dense feed-forward and
 latent-attention layers (compressed rows of width 128) with a routed feed-forward (32 experts of a
 sixteenth of the dense width plus 4 identity experts in 4 groups of which 2 are kept, 4 chosen, a shared
-expert of a quarter); the transformer has full causal attention and a SwiGLU feed-forward. Prints one
+expert of a quarter); the Surevik stack is window attention (the window is the others' chunk) with a routed
+feed-forward of the same sizes in every layer (32 clamped gated experts of a sixteenth of the dense width, 4
+chosen, a gated shared expert of a quarter), its second and third layer run twice, so that it has as many
+layer runs as the others have layers; the transformer has full causal attention and a SwiGLU feed-forward. Prints one
 JSON line. Per-kernel times come from running this under ``rocprofv3 --kernel-trace --stats``.
 """
 from __future__ import annotations
@@ -72,6 +75,20 @@ def telurax_config(s: dict):
                                    "shared": {"ff": s["ff"] // 4}}})
     return config_from_dict({"architecture": "Telurax", "vocab": s["vocab"], "width": s["width"], "norm": {"eps": 1e-5},
                              "embedding": {"scale": 1.0}, "logit_scale": 1.0, "layers": layers}, name="telurax-bench")
+
+
+def surevik_config(s: dict):
+    from .models.hybrid import config_from_dict
+
+    layer = {"type": "attention",
+             "mixer": {"heads": s["heads"], "kv_heads": s["kv"], "dim": s["dim"], "vdim": s["dim"], "scale": s["dim"] ** -0.5,
+                       "mask": {"size": s["chunk"]}, "rot": {"dims": s["dim"] // 2, "base": 10000.0}},
+             "mlp": {"kind": "moe", "expert": {"ff": s["ff"] // 16, "limit": 7.0}, "router": {"experts": 32, "top": 4},
+                     "shared": {"ff": s["ff"] // 4, "limit": 7.0}}}
+    return config_from_dict({"architecture": "Surevik", "vocab": s["vocab"], "width": s["width"], "norm": {"eps": 1e-6},
+                             "embedding": {"scale": s["width"] ** 0.5}, "residual_mult": 0.5,
+                             "layers": [layer] * (s["layers"] - 2), "loop": {"start": 1, "stop": 3, "times": 2}},
+                            name="surevik-bench")
 
 
 def transformer_config(s: dict):
@@ -143,6 +160,8 @@ def run(a) -> int:
                 model = HybridModel.random_init(hybrid_config(s), dev, seed=1)
             elif kind == "telurax":
                 model = HybridModel.random_init(telurax_config(s), dev, seed=1)
+            elif kind == "surevik":
+                model = HybridModel.random_init(surevik_config(s), dev, seed=1)
             else:
                 model = TransformerModel.random_init(transformer_config(s), dev, seed=1)
             row[kind] = _measure(model, a.hybrid_prompt, a.hybrid_batch, a.hybrid_new, a.steps, a.warmup, phases)
@@ -153,9 +172,10 @@ def run(a) -> int:
             k = ph + "_tokens_per_s"
             if all(k in row.get(m, {}) for m in ("nidozen", "llama")):
                 row[ph + "_ratio"] = row["nidozen"][k] / row["llama"][k]
-            for other in ("nidozen", "llama"):
-                if all(k in row.get(m, {}) for m in ("telurax", other)):
-                    row[f"{ph}_telurax_over_{other}"] = row["telurax"][k] / row[other][k]
+            for mine, others in (("telurax", ("nidozen", "llama")), ("surevik", ("telurax", "nidozen", "llama"))):
+                for other in others:
+                    if all(k in row.get(m, {}) for m in (mine, other)):
+                        row[f"{ph}_{mine}_over_{other}"] = row[mine][k] / row[other][k]
         res["sizes"][name] = row
     print(json.dumps(res))
     if a.out:

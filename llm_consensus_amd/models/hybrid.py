@@ -789,8 +789,11 @@ class HybridModel:
                 kw["router"] = lin(torch.cat(rows, 0), pad=True)
                 ups = torch.stack([torch.cat([load(f + f"e{j}.gate"), load(f + f"e{j}.up")], 0) for j in range(e.experts)])
                 downs = torch.stack([load(f + f"e{j}.down") for j in range(e.experts)])
-                if dt == torch.bfloat16 and c.hidden_size % 64 == 0 and e.ff % 64 == 0:
-                    kw["experts_up"] = ops.ExpertWeights.from_dense(ups, dev)
+                if dt == torch.bfloat16 and c.hidden_size % 64 == 0 and e.ff % 64 == 0 and dev.type == "cuda":
+                    # depths the MFMA kernels take: fragment order per expert, 16-row tiles alternating gate / up so
+                    # that the gated unit is the product's epilogue
+                    ups = torch.stack([ops.interleave_gate_up(load(f + f"e{j}.gate"), load(f + f"e{j}.up")) for j in range(e.experts)])
+                    kw["experts_up"] = ops.ExpertWeights.from_dense(ups, dev, swiglu=True)
                     kw["experts_down"] = ops.ExpertWeights.from_dense(downs, dev)
                 else:
                     kw["experts_up"], kw["experts_down"] = ups.to(dt).contiguous(), downs.to(dt).contiguous()
@@ -1030,11 +1033,16 @@ class HybridModel:
             shared = ops.linear(act, L.shared_down, out_f32=True)
             gate = su[:, 2 * sf + e.experts:2 * sf + e.experts + 1]
         ids, wts = ops.route_grouped(z, None, e.top, 1, 1, 1.0, score="sigmoid")
-        offsets, sorted_src, slot_of = ops.moe_sort(ids, e.experts)
         rows = ids.numel()
-        gu = ops.grouped_linear(xa, sorted_src, offsets, L.experts_up, torch.float32, rows)
-        act = ops.glu_clamped(gu, 0, e.ff, e.ff, e.limit, self.dtype, slot_of=slot_of.view(-1), wts=wts.view(-1),
-                              slope=des.glu_slope, shift=des.glu_shift)
+        if isinstance(L.experts_up, ops.ExpertWeights):     # (bf16, MFMA depths: the gated unit is the product's epilogue)
+            offsets, sorted_src, slot_of, sorted_wts = ops.moe_sort(ids, e.experts, wts)
+            act = ops.grouped_linear(xa, sorted_src, offsets, L.experts_up, self.dtype, rows,
+                                     glu_clamp=(sorted_wts, e.limit, des.glu_slope, des.glu_shift))
+        else:
+            offsets, sorted_src, slot_of = ops.moe_sort(ids, e.experts)
+            gu = ops.grouped_linear(xa, sorted_src, offsets, L.experts_up, torch.float32, rows)
+            act = ops.glu_clamped(gu, 0, e.ff, e.ff, e.limit, self.dtype, slot_of=slot_of.view(-1), wts=wts.view(-1),
+                                  slope=des.glu_slope, shift=des.glu_shift)
         ye = ops.grouped_linear(act, None, offsets, L.experts_down, torch.float32, rows)
         return ops.moe_mix(ye, slot_of, ids, None, xa, e.experts, shared, gate)
 

@@ -1233,27 +1233,56 @@ def route_grouped(z: torch.Tensor, correction: Optional[torch.Tensor], top: int,
     return ids, wts
 
 
-def moe_sort(ids: torch.Tensor, n: int):
+def moe_sort(ids: torch.Tensor, n: int, wts: Optional[torch.Tensor] = None):
     """``moe_permute`` for any number of experts (one block, counting sort): (offsets int32 [n+1],
-    sorted_src int32 [T*k], slot_of int32 [T*k])."""
+    sorted_src int32 [T*k], slot_of int32 [T*k]); with ``wts`` (fp32 [T, k]) also the weights in sorted
+    order, fp32 [T*k], as a fourth result."""
     if not ids.is_cuda:
-        return moe_permute(ids, n)
+        offsets, sorted_src, slot_of = moe_permute(ids, n)
+        if wts is None:
+            return offsets, sorted_src, slot_of
+        sw = torch.zeros(ids.numel(), dtype=torch.float32)
+        sw[slot_of.long()] = wts.reshape(-1).float()
+        return offsets, sorted_src, slot_of, sw
     T, topk = ids.shape
     dev = ids.device
     offsets = torch.empty(n + 1, dtype=torch.int32, device=dev)
     sorted_src = torch.empty(T * topk, dtype=torch.int32, device=dev)
     slot_of = torch.empty(T * topk, dtype=torch.int32, device=dev)
-    _hip().call("lc_moe_sort", ids.data_ptr(), T, topk, n, offsets.data_ptr(), sorted_src.data_ptr(), slot_of.data_ptr())
-    return offsets, sorted_src, slot_of
+    sw = torch.empty(T * topk, dtype=torch.float32, device=dev) if wts is not None else None
+    if wts is not None and (wts.dtype != torch.float32 or wts.numel() != ids.numel() or not wts.is_contiguous()):
+        raise ValueError("moe_sort: fp32 weights, one per (token, choice) pair")
+    _hip().call("lc_moe_sort", ids.data_ptr(), T, topk, n, offsets.data_ptr(), sorted_src.data_ptr(), slot_of.data_ptr(),
+                _hip().ptr(wts), _hip().ptr(sw))
+    return (offsets, sorted_src, slot_of) if wts is None else (offsets, sorted_src, slot_of, sw)
 
 
 def grouped_linear(x: torch.Tensor, row_index: Optional[torch.Tensor], offsets: torch.Tensor, W,
-                   out_dtype: torch.dtype, rows: int, relu2_epi: bool = False) -> torch.Tensor:
+                   out_dtype: torch.dtype, rows: int, relu2_epi: bool = False, glu_clamp=None) -> torch.Tensor:
     """Per-expert products over expert-sorted rows: position p in [offsets[e], offsets[e+1]) gives
     W[e] x[row_index[p]] (x[p] without an index); ``relu2_epi``: square of relu. W is either a
     row-major tensor [E, N, K] of any shape and type (fp32 accumulation on the vector ALUs) or
     packed ``ExpertWeights`` (bf16 activations, the grouped MFMA kernels: one panel per expert for a
-    few hundred rows, 128 x 128 tiles beyond). Positions of experts >= E are left unwritten."""
+    few hundred rows, 128 x 128 tiles beyond). Positions of experts >= E are left unwritten.
+    ``glu_clamp`` = (row_scale fp32 [rows] or None, limit, slope, shift), packed weights marked ``swiglu``
+    only (16-row tiles alternate gate / up, ``interleave_gate_up``): the clamped gated unit of the product,
+    scaled per sorted row, as the epilogue; the result is bf16 [rows, N / 2]."""
+    if glu_clamp is not None:
+        if not (isinstance(W, ExpertWeights) and W.swiglu and x.is_cuda and W.n % 32 == 0):
+            raise ValueError("grouped_linear: the gated epilogue takes packed gate / up tiles on the GPU")
+        if x.dtype != torch.bfloat16 or x.shape[1] != W.k or not x.is_contiguous() or out_dtype != torch.bfloat16:
+            raise ValueError("grouped_linear: packed experts take contiguous bf16 activations of their depth")
+        scale, limit, slope, shift = glu_clamp
+        if scale is not None and (scale.dtype != torch.float32 or scale.numel() < rows):
+            raise ValueError("grouped_linear: one fp32 scale per sorted row")
+        y = torch.empty(rows, W.n // 2, dtype=torch.bfloat16, device=x.device)
+        gg = "lc_gemm_panel_grouped_glu" if rows <= MOE_PANEL_MAX_ROWS else "lc_gemm_grouped_glu"
+        _hip().call(gg, W.data.data_ptr(), W.data[0].numel(), x.data_ptr(), _hip().ptr(row_index), offsets.data_ptr(),
+                    W.data.shape[0], y.data_ptr(), int(rows), W.n, W.k, W.n_pad, W.n // 2, _hip().ptr(scale), float(limit),
+                    float(slope), float(shift))
+        return y
+    if isinstance(W, ExpertWeights) and W.swiglu:
+        raise ValueError("grouped_linear: interleaved gate / up tiles need the gated epilogue")
     if isinstance(W, ExpertWeights) and W.data.dim() == 3:
         W = W.data                                    # CPU: [E, N, K]
     if not x.is_cuda:

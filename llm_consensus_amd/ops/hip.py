@@ -34,6 +34,8 @@ _SIGNATURES = {
     "lc_gemm256_splitk": [_P, _P, _P, _I, _I, _I, _I, _I, _I, _P],
     "lc_gemm256_grouped": [_P, _L, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _P],
     "lc_gemm_panel_grouped": [_P, _L, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _P],
+    "lc_gemm_grouped_glu": [_P, _L, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _P, _F, _F, _F, _P],
+    "lc_gemm_panel_grouped_glu": [_P, _L, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _P, _F, _F, _F, _P],
     "lc_rope_kv_write": [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P, _I, _P, _P],
     "lc_attn_prefill": [_P, _I, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _P],
     "lc_attn_decode": [_P, _I, _P, _P, _P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _I, _I, _I, _P],
@@ -78,7 +80,7 @@ _SIGNATURES = {
     "lc_rope_pairs_write": [_P, _I, _P, _P, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _P],
     # routed feed-forwards of hybrid decoders (hybrid_moe.hip)
     "lc_route_grouped": [_P, _I, _P, _I, _I, _I, _I, _I, _F, _I, _P, _P, _P],
-    "lc_moe_sort": [_P, _I, _I, _I, _P, _P, _P, _P],
+    "lc_moe_sort": [_P, _I, _I, _I, _P, _P, _P, _P, _P, _P],
     "lc_gemm_any_grouped": [_P, _I, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _P],
     "lc_moe_mix": [_P, _P, _P, _P, _P, _I, _P, _P, _I, _P, _I, _I, _I, _I, _P],
 }

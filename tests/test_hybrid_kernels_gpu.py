@@ -445,3 +445,24 @@ def test_expert_mix_without_weights_under_a_gated_shared_expert():
     got = ops.moe_mix(ye.to(DEV), slot_of, ids.to(DEV), None, h.to(DEV), E, shared.to(DEV), wide.to(DEV)[:, 4:5])
     want = ye[slot_of.cpu().long()].view(T, top, d).sum(1) + torch.sigmoid(wide[:, 4:5]) * shared
     torch.testing.assert_close(got.cpu(), want, atol=1e-5, rtol=1e-5)
+
+
+@pytest.mark.parametrize("T,top,E,d,ff", [(5, 2, 3, 64, 64), (100, 3, 6, 128, 192), (400, 4, 9, 64, 128), (33, 1, 40, 64, 32)])
+def test_clamped_gated_experts_as_the_epilogue_of_the_packed_product(T, top, E, d, ff):
+    """The gate | up product of every expert on the MFMA kernels (one panel per expert for few rows, tiles beyond) with
+    the clamped gated unit and the per-row scale in its epilogue, against the plain product and unit."""
+    g = torch.Generator().manual_seed(T + E)
+    x = torch.randn(T, d, generator=g).to(torch.bfloat16)
+    gate = (torch.randn(E, ff, d, generator=g) * 2 / d ** 0.5).to(torch.bfloat16)
+    up = (torch.randn(E, ff, d, generator=g) * 2 / d ** 0.5).to(torch.bfloat16)
+    ids = torch.stack([torch.randperm(E, generator=g)[:top] for _ in range(T)]).to(torch.int32)
+    wts = torch.rand(T, top, generator=g)
+    offsets, src, slot_of, sw = ops.moe_sort(ids.to(DEV), E, wts.to(DEV))
+    torch.testing.assert_close(sw.cpu()[slot_of.cpu().long()], wts.reshape(-1))
+    W = ops.ExpertWeights.from_dense(torch.stack([ops.interleave_gate_up(gate[e], up[e]) for e in range(E)]), DEV, swiglu=True)
+    got = ops.grouped_linear(x.to(DEV), src, offsets, W, torch.bfloat16, T * top, glu_clamp=(sw, 0.6, 1.702, 1.0))
+    plain = ref.grouped_linear(x, src.cpu(), offsets.cpu(), torch.cat([gate, up], 1), torch.float32, T * top)
+    want = ref.glu_clamped(plain, 0, ff, ff, 0.6, 1.702, 1.0, slot_of.cpu(), wts.reshape(-1), torch.float32, T * top)
+    torch.testing.assert_close(got.float().cpu(), want, atol=2e-2, rtol=2e-2)
+    with pytest.raises(ValueError):
+        ops.grouped_linear(x.to(DEV), src, offsets, W, torch.float32, T * top)

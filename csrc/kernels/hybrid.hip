@@ -5,6 +5,9 @@
 // (gemm*.hip: bf16, K a multiple of 64) do not take, including every product of the true-fp32
 // mode. Everything a recurrence or a softmax touches is fp32; only tensors that feed the next
 // matrix product are written in the activation type (bf16 or fp32, a launch-time flag).
+// Pre-norm designs add: a residual step fused with a per-coordinate RMS norm or with a Dynamic Tanh
+// norm, latent attention's cached row, matrix memories, per-head products, gated units (plain and
+// clamped), and attention whose values are its keys before they rotate in neighbouring pairs.
 //
 // A step's sequences are described by cu_q [B+1] (row ranges), positions [T] and slots [B]
 // (state slot of the sequence; < 0: padding row of a recorded step, skipped). A sequence whose

@@ -219,7 +219,7 @@ class HybridConfig:
 
     @property
     def looped(self) -> bool:
-        return self.loop[2] != 1 or self.loop[1] > self.loop[0]
+        return self.loop[1] > self.loop[0]          # (an empty range loops over nothing, whatever its count)
 
     @property
     def runs(self) -> Tuple[Tuple[int, bool], ...]:
@@ -272,8 +272,8 @@ class HybridConfig:
         known = self.design.mixers
         start, stop, times = self.loop
         if self.looped:
-            if not (0 <= start < stop <= len(self.layers)) or times < 1:
-                raise ValueError(f"{self.name}: loop: 0 <= start < stop <= layers and times >= 1 are needed")
+            if not (0 <= start and stop <= len(self.layers)) or times < 1:
+                raise ValueError(f"{self.name}: loop: 0 <= start, stop <= layers and times >= 1 are needed")
             if any(l.kv_from >= 0 for l in self.layers):
                 raise ValueError(f"{self.name}: looped layers and shared keys (kv_from) do not combine")
         if self.design.pos_base > 0 and self.hidden_size % 2:

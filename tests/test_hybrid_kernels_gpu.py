@@ -378,7 +378,7 @@ def test_dynamic_tanh_residual_step(dt, T, d):
 
 
 @pytest.mark.parametrize("dt", ACTS)
-@pytest.mark.parametrize("H,G,D,rot,window", [(4, 2, 32, 8, 7), (3, 3, 48, 48, 40), (2, 1, 16, 0, 5), (5, 1, 7, 6, 3), (6, 2, 64, 32, 100)])
+@pytest.mark.parametrize("H,G,D,rot,window", [(4, 2, 32, 8, 7), (3, 3, 48, 48, 40), (2, 1, 16, 0, 5), (5, 1, 7, 6, 3), (6, 3, 64, 16, 100)])
 def test_rotary_pairs_keys_as_values_and_window_attention(dt, H, G, D, rot, window):
     g = torch.Generator().manual_seed(H * 100 + D)
     lens, starts = [37, 70, 1, 1], [0, 130, 55, 3]          # two portions (one continuing at place 130), two decoded tokens

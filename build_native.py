@@ -96,7 +96,7 @@ def build_selftest(sanitize: str = "address,undefined") -> Path:
 KERNEL_GROUPS = {
     "base": ["device_runtime.hip", "elementwise.hip", "gemm.hip", "gemm256.hip", "gemm256w.hip", "gemm_panel.hip",
              "kgemm.hip", "sampling.hip"],
-    "hybrid": ["hybrid.hip", "hybrid_moe.hip"],
+    "hybrid": ["hybrid.hip", "hybrid_moe.hip", "hybrid_streams.hip"],
 }
 
 

@@ -674,6 +674,12 @@ __global__ __launch_bounds__(256) void rope_pairs_write_kernel(
 // off when 0). Per tile of 64 keys: lane j scores key lo + 64 * tile + j in fp32 (q from LDS),
 // online softmax across the wave, then the lanes split the value columns and walk the tile's
 // keys (weights and cache rows from LDS). Serves prompt portions and single decoded tokens.
+// Options: key / value rows may be column blocks of wider cache rows (row strides k_ld / v_ld); ``softcap`` > 0
+// bounds the scaled score s to softcap * tanh(s / softcap); ``sink``: a silent extra key of score 0 without a value
+// joins the softmax (the running maximum starts at 0 and the running sum at 1); ``vh0`` >= 0: the head's weights are
+// applied to the ``nvh`` value heads vh0 .. vh0 + nvh - 1 side by side instead of its own group's (designs that
+// mix the heads' weights afterwards need every head's weights on every value head). Output row (t, h) has ``o_ld``
+// columns, written from column ``o_col0`` on.
 constexpr int kMaxVCols = 8;   // value width up to 512
 
 template <bool CF32, bool AF32>
@@ -681,7 +687,7 @@ __global__ __launch_bounds__(256) void attn_masked_kernel(
     const float* __restrict__ q, const void* __restrict__ kc, const void* __restrict__ vc,
     const int32_t* __restrict__ block_tables, int MB, const int32_t* __restrict__ row_seq,
     const int32_t* __restrict__ positions, void* __restrict__ out, int H, int G, int D, int Dv, int BS, float scale,
-    int chunk, int window) {
+    int chunk, int window, int k_ld, int v_ld, float softcap, int sink, int vh0, int nvh, int o_ld, int o_col0) {
   extern __shared__ float lds[];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int t = blockIdx.x;
@@ -701,10 +707,18 @@ __global__ __launch_bounds__(256) void attn_masked_kernel(
   const int32_t* table = block_tables + static_cast<size_t>(seq) * MB;
   const typename Act<CF32>::type* kbase = static_cast<const typename Act<CF32>::type*>(kc);
   const typename Act<CF32>::type* vbase = static_cast<const typename Act<CF32>::type*>(vc);
-  float m = -INFINITY, l = 0.f;
+  float m = sink ? 0.f : -INFINITY, l = sink ? 1.f : 0.f;
   float acc[kMaxVCols];
+  int vcol[kMaxVCols], voff[kMaxVCols];            // a lane's value columns: column inside the head, row offset of the head's plane
+  const int ncols = nvh * Dv;
 #pragma unroll
-  for (int i = 0; i < kMaxVCols; ++i) acc[i] = 0.f;
+  for (int i = 0; i < kMaxVCols; ++i) {
+    acc[i] = 0.f;
+    const int c = lane + 64 * i;
+    const int vh = c / Dv;
+    vcol[i] = c - vh * Dv;
+    voff[i] = vh0 < 0 ? 0 : (vh0 + vh - g) * BS;
+  }
   __syncthreads();
   for (int j0 = lo; j0 <= p; j0 += 64) {
     const int j = j0 + lane;
@@ -713,9 +727,9 @@ __global__ __launch_bounds__(256) void attn_masked_kernel(
     int crow = 0;
     if (valid) {
       crow = (table[j / BS] * G + g) * BS + (j % BS);
-      const typename Act<CF32>::type* kr = kbase + static_cast<size_t>(crow) * D;
+      const typename Act<CF32>::type* kr = kbase + static_cast<size_t>(crow) * k_ld;
       float dot = 0.f;
-      if (!CF32 && D % 8 == 0) {
+      if (!CF32 && D % 8 == 0 && k_ld % 8 == 0) {
         // a bf16 key row in 16-byte pieces (rows start on 16-byte borders when D is a multiple of 8)
         const u32x4* kv = reinterpret_cast<const u32x4*>(kr);
         for (int c = 0; c < D / 8; ++c) {
@@ -728,7 +742,7 @@ __global__ __launch_bounds__(256) void attn_masked_kernel(
       } else {
         for (int d = 0; d < D; ++d) dot += qs[d] * Act<CF32>::load(kr, d);
       }
-      s = dot;
+      s = softcap > 0.f ? softcap * tanhf(dot / softcap) : dot;
     }
     const float mt = fmaxf(m, wave_max(s));
     const float pj = valid ? expf(s - mt) : 0.f;
@@ -742,10 +756,11 @@ __global__ __launch_bounds__(256) void attn_masked_kernel(
 #pragma unroll
     for (int i = 0; i < kMaxVCols; ++i) {
       const int c = lane + 64 * i;
-      if (c < Dv) {
+      if (c < ncols) {
         float a = acc[i] * corr;
 #pragma unroll 8                                    // eight value loads in flight at a time
-        for (int jj = 0; jj < n; ++jj) a += ps[jj] * Act<CF32>::load(vbase, static_cast<size_t>(rows[jj]) * Dv + c);
+        for (int jj = 0; jj < n; ++jj)
+          a += ps[jj] * Act<CF32>::load(vbase, static_cast<size_t>(rows[jj] + voff[i]) * v_ld + vcol[i]);
         acc[i] = a;
       }
     }
@@ -755,7 +770,7 @@ __global__ __launch_bounds__(256) void attn_masked_kernel(
 #pragma unroll
   for (int i = 0; i < kMaxVCols; ++i) {
     const int c = lane + 64 * i;
-    if (live && c < Dv) Act<AF32>::store(o, (static_cast<size_t>(t) * H + h) * Dv + c, acc[i] / l);
+    if (live && c < ncols) Act<AF32>::store(o, (static_cast<size_t>(t) * H + h) * o_ld + o_col0 + c, acc[i] / l);
   }
 }
 
@@ -770,6 +785,8 @@ __global__ __launch_bounds__(256) void attn_masked_kernel(
 //   (the 16 lanes of a row's keys reduce by shuffles), P through LDS into the A layout,
 //   O += P V    4 MFMAs per 16 value columns (B: v[key 4j + (l>>4)][col l&15]).
 // Row strides in LDS are padded so that the 16 rows of an operand fall into different banks.
+// The options of the row kernel (row strides, score cap, sink, value heads side by side) apply here too; the value
+// tile then holds nvh * Dv columns.
 constexpr int kTileMaxVT = 16;     // value width up to 256
 
 LC_DEVICE int lds_stride(int n, int want) { return n + ((want - n % 32 + 32) % 32); }
@@ -816,7 +833,7 @@ __global__ __launch_bounds__(256) void attn_tile_kernel(
     const float* __restrict__ q, const void* __restrict__ kc, const void* __restrict__ vc,
     const int32_t* __restrict__ block_tables, int MB, const int32_t* __restrict__ cu_q,
     const int32_t* __restrict__ positions, void* __restrict__ out, int H, int G, int D, int Dv, int BS, float scale,
-    int chunk, int window) {
+    int chunk, int window, int k_ld, int v_ld, float softcap, int sink, int vh0, int nvh, int o_ld, int o_col0) {
   extern __shared__ float lds[];
   const int b = blockIdx.z, h = blockIdx.y;
   const int q0 = cu_q[b], q1 = cu_q[b + 1];
@@ -825,12 +842,13 @@ __global__ __launch_bounds__(256) void attn_tile_kernel(
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int lr = lane & 15, lk = lane >> 4;
   const int g = h / (H / G);
-  const int DS = lds_stride(D, 4), VS = lds_stride(Dv, 16);
+  const int ncols = nvh * Dv;                               // value columns of the block: nvh heads side by side
+  const int DS = lds_stride(D, 4), VS = lds_stride(ncols, 16);
   float* Qs = lds;                                          // [4][16][DS]
   float* Ks = Qs + 64 * DS;                                 // [16][DS]
   float* Vs = Ks + 16 * DS;                                 // [16][VS]
   float* Ps = Vs + 16 * VS + wave * 16 * 17;                // [4][16][17]
-  const int nt = Dv / 16;
+  const int nt = ncols / 16;
   const int32_t* table = block_tables + static_cast<size_t>(b) * MB;
   // queries of the block's rows, scaled (rows past the portion: zero)
   for (int i = threadIdx.x; i < 64 * D; i += 256) {
@@ -850,15 +868,17 @@ __global__ __launch_bounds__(256) void attn_tile_kernel(
   const int wave_rows = max(0, min(16, nrows - 16 * wave));
   const int wave_lo = first_key(pw0), wave_hi = pw0 + wave_rows - 1;
   // staging: a tile is 16 keys x D (x Dv) elements = 2 D (2 Dv) units of 8; a thread owns up to two of each
-  const int ku = D / 8, vu = Dv / 8;
-  int kkey[2], kcol[2], vkey[2], vcol[2];
+  const int ku = D / 8, vu = ncols / 8;
+  int kkey[2], kcol[2], vkey[2], vcol[2], vhead[2], vin[2];
 #pragma unroll
   for (int i = 0; i < 2; ++i) {
     const int u = threadIdx.x + 256 * i;
     kkey[i] = u < 16 * ku ? u / ku : -1;
     kcol[i] = (u % ku) * 8;
     vkey[i] = u < 16 * vu ? u / vu : -1;
-    vcol[i] = (u % vu) * 8;
+    vcol[i] = (u % vu) * 8;                                 // column in the tile; inside its head: vin
+    vhead[i] = vh0 < 0 ? g : vh0 + vcol[i] / Dv;
+    vin[i] = vcol[i] % Dv;
   }
   Raw8<CF32> kr[2], vr[2];
   auto fetch = [&](int j0) {
@@ -867,17 +887,17 @@ __global__ __launch_bounds__(256) void attn_tile_kernel(
       const int jk = j0 + kkey[i], jv = j0 + vkey[i];
       const bool kon = kkey[i] >= 0 && jk <= hi, von = vkey[i] >= 0 && jv <= hi;
       const size_t krow = kon ? (static_cast<size_t>(table[jk / BS]) * G + g) * BS + jk % BS : 0;
-      const size_t vrow = von ? (static_cast<size_t>(table[jv / BS]) * G + g) * BS + jv % BS : 0;
-      kr[i] = load_raw8<CF32>(kc, krow * D + kcol[i], kon);
-      vr[i] = load_raw8<CF32>(vc, vrow * Dv + vcol[i], von);
+      const size_t vrow = von ? (static_cast<size_t>(table[jv / BS]) * G + vhead[i]) * BS + jv % BS : 0;
+      kr[i] = load_raw8<CF32>(kc, krow * k_ld + kcol[i], kon);
+      vr[i] = load_raw8<CF32>(vc, vrow * v_ld + vin[i], von);
     }
   };
   float m[4], l[4];
   f32x4 o[kTileMaxVT];
 #pragma unroll
   for (int r = 0; r < 4; ++r) {
-    m[r] = -INFINITY;
-    l[r] = 0.f;
+    m[r] = sink ? 0.f : -INFINITY;
+    l[r] = sink ? 1.f : 0.f;
   }
 #pragma unroll
   for (int t = 0; t < kTileMaxVT; ++t) o[t] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -907,7 +927,8 @@ __global__ __launch_bounds__(256) void attn_tile_kernel(
       const int row = 4 * lk + r;
       const int prow = pw0 + row;
       const bool valid = row < wave_rows && j <= prow && j >= first_key(prow);
-      const float sv = valid ? sacc[0][r] + sacc[1][r] : -INFINITY;
+      const float sraw = sacc[0][r] + sacc[1][r];
+      const float sv = valid ? (softcap > 0.f ? softcap * tanhf(sraw / softcap) : sraw) : -INFINITY;
       float mt = sv;
 #pragma unroll
       for (int off = 8; off > 0; off >>= 1) mt = fmaxf(mt, __shfl_xor(mt, off, 64));
@@ -953,7 +974,8 @@ __global__ __launch_bounds__(256) void attn_tile_kernel(
       for (int r = 0; r < 4; ++r) {
         const int row = 4 * lk + r;
         if (row < wave_rows)
-          Act<AF32>::store(dst, (static_cast<size_t>(row0 + 16 * wave + row) * H + h) * Dv + t * 16 + lr, o[t][r] / l[r]);
+          Act<AF32>::store(dst, (static_cast<size_t>(row0 + 16 * wave + row) * H + h) * o_ld + o_col0 + t * 16 + lr,
+                           o[t][r] / l[r]);
       }
     }
   }
@@ -1020,13 +1042,16 @@ __global__ __launch_bounds__(256) void gemm_any_kernel(const void* __restrict__ 
 // ---------------------------------------------------------------- per-head products
 // C[m, h, :] = W[h] A[m, h, :] for H heads side by side: A [M, H*K] (row stride lda), W [H, N, K],
 // C [M, H*N]. The tiling of gemm_any_kernel with the head as the third grid dimension. With
-// ``gate`` [M, H] (row stride ld_gate) the head's outputs are scaled by sigmoid(gate[m, h]).
+// ``gate`` [M, H] (row stride ld_gate) the head's outputs are scaled by sigmoid(gate[m, h]); ``gate_full``: the gate
+// is [M, H*N], one logit per output. Head h's inputs start at column h * a_hs of A, its outputs at column h * c_hs
+// of C (row stride c_ld): heads may be column blocks of wider per-head rows on either side.
 // RPT rows per thread: a block covers 16 * RPT rows x 64 columns. Few rows (decode steps) take RPT = 1, which
 // spreads the same products over four times as many waves.
 template <bool AF32, bool WF32, bool CF32, int RPT>
 __global__ __launch_bounds__(256) void head_linear_kernel(const void* __restrict__ A, int lda, const void* __restrict__ W,
                                                           void* __restrict__ C, const float* __restrict__ gate,
-                                                          int ld_gate, int M, int H, int N, int K) {
+                                                          int ld_gate, int M, int H, int N, int K, int a_hs, int c_ld,
+                                                          int c_hs, int gate_full) {
   constexpr int KS = 32;                            // slab depth: per-head depths are short, so few, deep slabs
   constexpr int TM = 16 * RPT;
   constexpr int NA = TM * KS / 256, NW = 64 * KS / 256;
@@ -1035,7 +1060,7 @@ __global__ __launch_bounds__(256) void head_linear_kernel(const void* __restrict
   const int h = blockIdx.z;
   const int m0 = blockIdx.y * TM, n0 = blockIdx.x * 64;
   const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
-  const typename Act<AF32>::type* a = static_cast<const typename Act<AF32>::type*>(A) + static_cast<size_t>(h) * K;
+  const typename Act<AF32>::type* a = static_cast<const typename Act<AF32>::type*>(A) + static_cast<size_t>(h) * a_hs;
   const typename Act<WF32>::type* w = static_cast<const typename Act<WF32>::type*>(W) + static_cast<size_t>(h) * N * K;
   float acc[RPT][4] = {};
   // the next slab's elements are loaded into registers before the current one is multiplied, so the
@@ -1088,11 +1113,13 @@ __global__ __launch_bounds__(256) void head_linear_kernel(const void* __restrict
   for (int i = 0; i < RPT; ++i) {
     const int r = m0 + ty * RPT + i;
     if (r >= M) continue;
-    const float g = gate != nullptr ? sigmoidf_(gate[static_cast<size_t>(r) * ld_gate + h]) : 1.f;
+    const float g = gate != nullptr && !gate_full ? sigmoidf_(gate[static_cast<size_t>(r) * ld_gate + h]) : 1.f;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int col = n0 + tx * 4 + j;
-      if (col < N) Act<CF32>::store(c, (static_cast<size_t>(r) * H + h) * N + col, acc[i][j] * g);
+      if (col >= N) continue;
+      const float ge = gate_full ? sigmoidf_(gate[static_cast<size_t>(r) * ld_gate + h * N + col]) : g;
+      Act<CF32>::store(c, static_cast<size_t>(r) * c_ld + static_cast<size_t>(h) * c_hs + col, acc[i][j] * ge);
     }
   }
 }
@@ -1366,18 +1393,21 @@ LC_EXPORT int lc_latent_write(const void* proj, int ld, int col0, int R, const v
 }
 
 LC_EXPORT int lc_head_linear(const void* A, int a_f32, int lda, const void* W, int w_f32, void* C, int c_f32,
-                             const void* gate, int ld_gate, int M, int H, int N, int K, hipStream_t st) {
+                             const void* gate, int ld_gate, int M, int H, int N, int K, int a_hs, int c_ld, int c_hs,
+                             int gate_full, hipStream_t st) {
   if (M <= 0 || N <= 0 || H <= 0) return 0;
-  if (K <= 0 || lda < H * K || H > 65535 || (gate != nullptr && ld_gate < H)) return -1;
+  if (K <= 0 || a_hs < K || lda < (H - 1) * a_hs + K || H > 65535 || c_hs < N || c_ld < (H - 1) * c_hs + N) return -1;
+  if (gate != nullptr && ld_gate < (gate_full ? H * N : H)) return -1;
+  if (gate == nullptr && gate_full) return -1;
   const bool few = M <= 64;                          // decode steps: one row per thread, four times the blocks
   const dim3 grid((N + 63) / 64, few ? (M + 15) / 16 : (M + 63) / 64, H), block(256);
 #define LC_HL(A32, W32, C32)                                                                                       \
   if (few)                                                                                                         \
     head_linear_kernel<A32, W32, C32, 1><<<grid, block, 0, st>>>(A, lda, W, C, static_cast<const float*>(gate), ld_gate, \
-                                                                 M, H, N, K);                                      \
+                                                                 M, H, N, K, a_hs, c_ld, c_hs, gate_full);         \
   else                                                                                                             \
     head_linear_kernel<A32, W32, C32, 4><<<grid, block, 0, st>>>(A, lda, W, C, static_cast<const float*>(gate), ld_gate, \
-                                                                 M, H, N, K)
+                                                                 M, H, N, K, a_hs, c_ld, c_hs, gate_full)
   const int sel = (a_f32 ? 4 : 0) | (w_f32 ? 2 : 0) | (c_f32 ? 1 : 0);
   switch (sel) {
     case 0: LC_HL(false, false, false); break;
@@ -1432,9 +1462,12 @@ LC_EXPORT int lc_qkv_prep(const void* qkv, int ld, const void* qn, const void* k
 
 LC_EXPORT int lc_attn_masked(const void* q, const void* kc, const void* vc, int cache_f32, const void* block_tables,
                              int MB, const void* row_seq, const void* positions, void* out, int act_f32, int T, int H,
-                             int G, int D, int Dv, int BS, float scale, int chunk, int window, hipStream_t st) {
+                             int G, int D, int Dv, int BS, float scale, int chunk, int window, int k_ld, int v_ld,
+                             float softcap, int sink, int vh0, int nvh, int o_ld, int o_col0, hipStream_t st) {
   if (T <= 0) return 0;
-  if (H <= 0 || G <= 0 || H % G || D <= 0 || Dv <= 0 || Dv > 64 * kMaxVCols || BS <= 0 || MB <= 0) return -1;
+  if (H <= 0 || G <= 0 || H % G || D <= 0 || Dv <= 0 || BS <= 0 || MB <= 0) return -1;
+  if (nvh <= 0 || nvh * Dv > 64 * kMaxVCols || (vh0 < 0 && nvh != 1) || (vh0 >= 0 && vh0 + nvh > G)) return -1;
+  if (k_ld < D || v_ld < Dv || o_col0 < 0 || o_ld < o_col0 + nvh * Dv || softcap < 0.f) return -1;
   const size_t lds = 4 * static_cast<size_t>(D + 128) * sizeof(float);
   if (lds > 64 * 1024) return -1;
   const dim3 grid(T, (H + 3) / 4), block(256);
@@ -1442,7 +1475,7 @@ LC_EXPORT int lc_attn_masked(const void* q, const void* kc, const void* vc, int 
   attn_masked_kernel<C32, A32><<<grid, block, lds, st>>>(                                                       \
       static_cast<const float*>(q), kc, vc, static_cast<const int32_t*>(block_tables), MB,                      \
       static_cast<const int32_t*>(row_seq), static_cast<const int32_t*>(positions), out, H, G, D, Dv, BS, scale, \
-      chunk, window)
+      chunk, window, k_ld, v_ld, softcap, sink, vh0, nvh, o_ld, o_col0)
   if (cache_f32 && act_f32) LC_ATT(true, true);
   else if (cache_f32) LC_ATT(true, false);
   else if (act_f32) LC_ATT(false, true);
@@ -1456,11 +1489,16 @@ LC_EXPORT int lc_attn_masked(const void* q, const void* kc, const void* vc, int 
 LC_EXPORT int lc_attn_tile(const void* q, const void* kc, const void* vc, int cache_f32, const void* block_tables,
                            int MB, const void* cu_q, const void* positions, void* out, int act_f32, int n_seq,
                            int max_len, int H, int G, int D, int Dv, int BS, float scale, int chunk, int window,
+                           int k_ld, int v_ld, float softcap, int sink, int vh0, int nvh, int o_ld, int o_col0,
                            hipStream_t st) {
   if (n_seq <= 0 || max_len <= 0) return 0;
   if (H <= 0 || G <= 0 || H % G || D <= 0 || Dv <= 0 || BS <= 0 || MB <= 0) return -1;
-  if (D % 8 || Dv % 16 || Dv > 16 * kTileMaxVT || D > 256) return -2;
-  const int DS = D + ((4 - D % 32 + 32) % 32), VS = Dv + ((16 - Dv % 32 + 32) % 32);
+  if (nvh <= 0 || (vh0 < 0 && nvh != 1) || (vh0 >= 0 && vh0 + nvh > G)) return -1;
+  if (k_ld < D || v_ld < Dv || o_col0 < 0 || o_ld < o_col0 + nvh * Dv || softcap < 0.f) return -1;
+  const int NC = nvh * Dv;
+  // (16-byte loads of the staged tiles: rows and column blocks start on 16-byte borders)
+  if (D % 8 || Dv % 16 || NC > 16 * kTileMaxVT || D > 256 || k_ld % 8 || v_ld % 8) return -2;
+  const int DS = D + ((4 - D % 32 + 32) % 32), VS = NC + ((16 - NC % 32 + 32) % 32);
   const size_t lds = (static_cast<size_t>(80) * DS + 16 * VS + 4 * 16 * 17) * sizeof(float);
   if (lds > 64 * 1024) return -2;
   const dim3 grid((max_len + 63) / 64, H, n_seq), block(256);
@@ -1468,7 +1506,7 @@ LC_EXPORT int lc_attn_tile(const void* q, const void* kc, const void* vc, int ca
   attn_tile_kernel<C32, A32><<<grid, block, lds, st>>>(                                                         \
       static_cast<const float*>(q), kc, vc, static_cast<const int32_t*>(block_tables), MB,                      \
       static_cast<const int32_t*>(cu_q), static_cast<const int32_t*>(positions), out, H, G, D, Dv, BS, scale,   \
-      chunk, window)
+      chunk, window, k_ld, v_ld, softcap, sink, vh0, nvh, o_ld, o_col0)
   if (cache_f32 && act_f32) LC_TILE(true, true);
   else if (cache_f32) LC_TILE(true, false);
   else if (act_f32) LC_TILE(false, true);

@@ -2,9 +2,28 @@
 paged cache, latent attention over a cache of compressed rows, minGRU, gated linear attention or
 mLSTM -- around an fp32 residual stream.
 
-Three designs are served, told apart by ``architecture`` in ``config.json`` (``DESIGNS``); the file lists
+Four designs are served, told apart by ``architecture`` in ``config.json`` (``DESIGNS``); the file lists
 the layers (``layers[i].type``, ``.mixer`` sizes, ``.mlp``), and every size and constant comes from
 there or from a tensor's shape.
+
+Gizilorn (pre-norm, a residual of several parallel streams):
+
+* ``e = rms_norm(embed[token]) * w_e``; the residual is ``streams`` copies x_1 .. x_S of e. A sublayer reads
+  ``u = sum_s in[s] x_s`` through its RMS norm and writes all streams at once from the old ones,
+  ``x_t <- sum_s mix[s, t] x_s + out[t] y`` (``hc1`` for the mixer, ``hc2`` for the feed-forward); the model's
+  output is ``head . rms_norm(sum_s x_s)``;
+* ``attention``: biased q / k / v projections; q and k turn over their first ``rot.dims`` coordinates (i with
+  i + dims / 2), the values over their WHOLE width by their own position and are cached so; scores are scaled,
+  then capped (``softcap * tanh(s / softcap)``); a window of ``mask.size`` positions; a softmax with one added to
+  its denominator; the heads' weights are mixed by ``talk`` [H, H] before they meet the values of the head's own
+  group; each head's result turns back by the row's position; ``W_o``;
+* ``latent_attention``: a query head is [dim plain | rot_dim turned] coordinates; the cached row per token is the
+  RMS-normed compressed row (``kv_rank``) beside ONE turned key part (``rot_dim``, neighbouring pairs) that all
+  heads share; keys and values are linear maps of the compressed row (moved to the query and the output side as
+  for Telurax); a window; a plain softmax; the heads' results are gated coordinate by coordinate with
+  ``sigmoid(W_g h)``; ``kv_from: j`` reads layer j's cached rows (no down-projection of its own);
+* feed-forward: ``down(xielu(up h + b) ) + b`` with xIELU ``softplus(p) z^2 + z/2`` above zero and
+  ``(1/2 + softplus(q)) (exp(z) - 1 - z) + z/2`` below.
 
 Surevik (pre-norm, Dynamic Tanh norms):
 
@@ -88,12 +107,21 @@ class Design:
     pre_norm: bool = False          # norms with a weight per coordinate on the sublayer INPUTS (else: one-gain norms on the outputs)
     norm_offset: float = 0.0        # stored norm weights are offsets from this value
     pos_base: float = 0.0           # > 0: a sinusoidal position vector of this base is added to the embedding
-    dense_ff: str = "relu2"         # dense feed-forward: down(relu(up x)^2) | "glu_relu": down(relu(gate x) * up x) | "": none
+    dense_ff: str = "relu2"         # dense feed-forward: down(relu(up x)^2) | "glu_relu": down(relu(gate x) * up x) |
+                                    # "xielu": down(xielu(up x + b)) + b with the activation's two numbers in ``mlp.act`` | "": none
     norm: str = "rms"               # "dyt": Dynamic Tanh, tanh(alpha x) * w + b (tensors <name>, <name>.b, <name>.alpha)
     tied_head: bool = False         # logits from the embedding table (no ``head`` tensor)
     attention: str = "normed"       # what the ``attention`` mixer is: "normed" (biases, whole-projection q / k norms,
                                     # rotate-half pairs, unit-RMS values, ``mask.size`` = chunk) | "keys_as_values" (no
                                     # biases or norms, values = the un-rotated keys, neighbouring pairs, ``mask.size`` = window)
+                                    # | "talking" (biased q / k / v, rotate-half pairs on q and k, values turned by their own
+                                    # position, capped scores, ``mask.size`` = window, a sink in the softmax, the heads'
+                                    # weights mixed by a matrix)
+    latent: str = "plain"           # latent attention: "plain" (no positions, all earlier rows, a gate per head) | "rotary" (a
+                                    # turned key part shared by all heads beside the compressed row, a window, a gate per
+                                    # output coordinate, ``kv_from``)
+    embed_norm: bool = False        # an RMS norm (tensor ``embed.norm``) on the embedding rows
+    hyper: bool = False             # the residual is ``streams`` parallel streams (tensors ``<layer>.hc<q>.{in,out,mix}``)
     routed_ff: str = "grouped_relu2"    # "sigmoid_clamped": sigmoid scores, weight on the expert's input, clamped gated experts
     # constants of the clamped gated unit g * sigmoid(slope g) * (u + shift)
     glu_slope: float = 1.702
@@ -106,6 +134,8 @@ DESIGNS: Dict[str, Design] = {
                       dense_ff="glu_relu"),
     "Surevik": Design("Surevik", ("attention",), pre_norm=True, dense_ff="", norm="dyt", tied_head=True,
                       attention="keys_as_values", routed_ff="sigmoid_clamped"),
+    "Gizilorn": Design("Gizilorn", ("attention", "latent_attention"), pre_norm=True, dense_ff="xielu", attention="talking",
+                       latent="rotary", embed_norm=True, hyper=True),
 }
 MIXERS = tuple(dict.fromkeys(m for d in DESIGNS.values() for m in d.mixers))
 
@@ -156,15 +186,24 @@ class LayerSpec:
     window: int = 0              # keys visible only this far back (0: all)
     rot_dims: int = 0
     rot_base: float = 10000.0
-    kv_from: int = -1            # attention: read this layer's keys and values (-1: own)
+    kv_from: int = -1            # attention / latent attention: read this layer's cached rows (-1: own)
     values_are_keys: bool = False    # attention: no norms, biases or value projection; neighbouring rotary pairs
+    # attention whose heads' weights are mixed: score cap (0: none), a softmax with one added to its denominator,
+    # values turned by their own position over their whole width (and the result turned back)
+    talk: bool = False
+    softcap: float = 0.0
+    sink: bool = False
+    rotate_values: bool = False
     # gla
     tau: float = 1.0
     rank: int = 0                # width of the decay's low-rank bottleneck (from the tensor's shape)
     # mingru
     width: int = 0
-    # latent attention: width of the cached compressed row
+    # latent attention: width of the cached compressed row; width of the turned key part cached beside it (0: none),
+    # which is also the turned part of every query head; a gate per output coordinate instead of one per head
     kv_rank: int = 0
+    rot_dim: int = 0
+    gate_full: bool = False
     # mlstm: soft cap of the gate logits (0: none)
     gate_cap: float = 0.0
     # feed-forward (0: none); ``moe``: a routed one instead of the dense one
@@ -174,6 +213,10 @@ class LayerSpec:
     @property
     def owns_kv(self) -> bool:
         return self.type == "attention" and self.kv_from < 0
+
+    @property
+    def owns_latent(self) -> bool:
+        return self.type == "latent_attention" and self.kv_from < 0
 
     @property
     def has_ff(self) -> bool:
@@ -195,7 +238,7 @@ class LayerSpec:
             return self.kv_heads * self.dim * (2 if self.rot_dims else 1)
         if self.owns_kv:
             return self.kv_heads * (self.dim + self.vdim)
-        return self.kv_rank if self.type == "latent_attention" else 0
+        return self.kv_rank + self.rot_dim if self.owns_latent else 0
 
 
 @dataclass(frozen=True)
@@ -212,6 +255,7 @@ class HybridConfig:
     logit_scale: float = 1.0
     residual_mult: float = 1.0      # every sublayer output is scaled by this before it joins the stream
     loop: Tuple[int, int, int] = (0, 0, 1)      # layers [start, stop) run ``times`` times in a row (times 1: no loop)
+    streams: int = 0                # parallel residual streams (designs with hyper-connections)
 
     @property
     def design(self) -> Design:
@@ -278,6 +322,8 @@ class HybridConfig:
                 raise ValueError(f"{self.name}: looped layers and shared keys (kv_from) do not combine")
         if self.design.pos_base > 0 and self.hidden_size % 2:
             raise ValueError(f"{self.name}: a sinusoidal position vector needs an even width")
+        if self.design.hyper and (not 1 <= self.streams <= ops.MAX_STREAMS or self.looped):
+            raise ValueError(f"{self.name}: 1..{ops.MAX_STREAMS} residual streams are needed, and no loop")
         for i, l in enumerate(self.layers):
             if l.type not in known:
                 raise ValueError(f"{self.name}: layer {i}: unknown mixer {l.type!r} (known: {', '.join(known)})")
@@ -285,6 +331,15 @@ class HybridConfig:
                 raise ValueError(f"{self.name}: layer {i}: heads, dim and vdim are needed")
             if l.type == "latent_attention" and (l.kv_rank <= 0 or l.kv_rank > 512):
                 raise ValueError(f"{self.name}: layer {i}: the attention kernels take a latent width of 1..512")
+            if l.type == "latent_attention" and (l.rot_dim % 2 or l.rot_dim < 0 or l.rot_dims != l.rot_dim or l.window < 0):
+                raise ValueError(f"{self.name}: layer {i}: the turned key part has an even width, and rot.dims equals it")
+            if l.type == "latent_attention" and l.kv_from >= 0:
+                src = self.layers[l.kv_from] if l.kv_from < i else None
+                if src is None or not src.owns_latent:
+                    raise ValueError(f"{self.name}: layer {i}: kv_from must name an earlier latent-attention layer with a "
+                                     f"down-projection of its own")
+                if (src.kv_rank, src.rot_dim, src.rot_base) != (l.kv_rank, l.rot_dim, l.rot_base):
+                    raise ValueError(f"{self.name}: layer {i}: kv_from layer {l.kv_from} has another latent width or rotation")
             if l.type == "mlstm" and (l.dim > 256 or l.gate_cap < 0):
                 raise ValueError(f"{self.name}: layer {i}: mLSTM takes dim <= 256 and a gate cap >= 0")
             if l.moe is not None:
@@ -310,6 +365,9 @@ class HybridConfig:
                     raise ValueError(f"{self.name}: layer {i}: rot.dims must be even and at most dim")
                 if l.vdim > 256:
                     raise ValueError(f"{self.name}: layer {i}: the attention kernel takes vdim <= 256")
+                if l.talk and (l.kv_from >= 0 or l.chunk or l.softcap < 0 or l.window < 0 or (l.rotate_values and l.vdim % 2)):
+                    raise ValueError(f"{self.name}: layer {i}: mixed heads take keys of their own, a cap >= 0, and values "
+                                     f"of even width when they turn")
                 if l.values_are_keys and (l.vdim != l.dim or l.kv_from >= 0 or l.chunk):
                     raise ValueError(f"{self.name}: layer {i}: values that are the keys have the keys' width (vdim = dim)")
                 if l.kv_from >= 0:
@@ -375,6 +433,21 @@ def config_from_dict(c: dict, name: str = "hybrid", tensor_shapes: Optional[Dict
                                     dim=int(m["dim"]), vdim=int(m.get("vdim", m["dim"])), scale=float(m["scale"]),
                                     window=int(mask.get("size", 0)), rot_dims=int(rot.get("dims", 0)),
                                     rot_base=float(rot.get("base", 10000.0)), values_are_keys=True, ff=ff, moe=moe))
+        elif t == "attention" and design.attention == "talking":
+            mask, rot = m.get("mask") or {}, m.get("rot") or {}
+            layers.append(LayerSpec(t, heads=int(m["heads"]), kv_heads=int(m.get("kv_heads", m["heads"])),
+                                    dim=int(m["dim"]), vdim=int(m.get("vdim", m["dim"])), scale=float(m["scale"]),
+                                    window=int(mask.get("size", 0)), rot_dims=int(rot.get("dims", 0)),
+                                    rot_base=float(rot.get("base", 10000.0)), talk=True, softcap=float(m.get("softcap", 0.0)),
+                                    sink=True, rotate_values=True, ff=ff))
+        elif t == "latent_attention" and design.latent == "rotary":
+            mask, rot = m.get("mask") or {}, m.get("rot") or {}
+            kvf = m.get("kv_from")
+            layers.append(LayerSpec(t, heads=int(m["heads"]), dim=int(m["dim"]), vdim=int(m.get("vdim", m["dim"])),
+                                    kv_rank=int(m["kv_rank"]), rot_dim=int(m.get("rot_dim", 0)), scale=float(m["scale"]),
+                                    window=int(mask.get("size", 0)), rot_dims=int(rot.get("dims", m.get("rot_dim", 0))),
+                                    rot_base=float(rot.get("base", 10000.0)), kv_from=-1 if kvf is None else int(kvf),
+                                    gate_full=True, ff=ff))
         elif t == "attention":
             mask, rot = m.get("mask") or {}, m.get("rot") or {}
             kvf = m.get("kv_from")
@@ -403,7 +476,7 @@ def config_from_dict(c: dict, name: str = "hybrid", tensor_shapes: Optional[Dict
                        max_position=int(c.get("max_position", 1 << 20)), model_type=arch.lower(), architecture=arch,
                        embed_scale=float((c.get("embedding") or {}).get("scale", 1.0)),
                        logit_scale=float(c.get("logit_scale", 1.0)), residual_mult=float(c.get("residual_mult", 1.0)),
-                       loop=_loop_of(c.get("loop")))
+                       loop=_loop_of(c.get("loop")), streams=int(c.get("streams", 1)) if design.hyper else 0)
     cfg.validate()
     return cfg
 
@@ -414,6 +487,14 @@ def config_to_dict(cfg: HybridConfig) -> dict:
         if l.type == "attention" and l.values_are_keys:
             m = {"heads": l.heads, "kv_heads": l.kv_heads, "dim": l.dim, "vdim": l.vdim, "scale": l.scale,
                  "mask": {"size": l.window}, "rot": {"dims": l.rot_dims, "base": l.rot_base}}
+        elif l.type == "attention" and l.talk:
+            m = {"heads": l.heads, "kv_heads": l.kv_heads, "dim": l.dim, "vdim": l.vdim, "scale": l.scale,
+                 "softcap": l.softcap, "mask": {"size": l.window}, "rot": {"dims": l.rot_dims, "base": l.rot_base}}
+        elif l.type == "latent_attention" and l.gate_full:
+            m = {"heads": l.heads, "dim": l.dim, "rot_dim": l.rot_dim, "vdim": l.vdim, "kv_rank": l.kv_rank, "scale": l.scale,
+                 "mask": {"size": l.window}, "rot": {"dims": l.rot_dims, "base": l.rot_base}}
+            if l.kv_from >= 0:
+                m["kv_from"] = l.kv_from
         elif l.type == "attention":
             m = {"heads": l.heads, "kv_heads": l.kv_heads, "dim": l.dim, "vdim": l.vdim, "scale": l.scale,
                  "mask": {"size": l.chunk} if not l.window else {"size": l.chunk, "window": l.window},
@@ -442,6 +523,9 @@ def config_to_dict(cfg: HybridConfig) -> dict:
         layers.append({"type": l.type, "mixer": m, "mlp": mlp})
     out = {"architecture": cfg.architecture, "vocab": cfg.vocab_size, "width": cfg.hidden_size,
            "norm": {"eps": cfg.rms_eps}, "layers": layers}
+    if cfg.design.hyper:
+        out["streams"] = cfg.streams
+        return out
     if cfg.design.pre_norm:
         out["embedding"] = {"scale": cfg.embed_scale}
     if cfg.design.pre_norm and not cfg.design.tied_head:
@@ -480,13 +564,29 @@ def param_shapes(cfg: HybridConfig) -> Dict[str, tuple]:
             out[name + ".b"], out[name + ".alpha"] = (d,), ()
     if cfg.looped:
         out["loop.in"] = (d, 2 * d)
+    if cfg.design.embed_norm:
+        out["embed.norm"] = (d,)
     for i, l in enumerate(cfg.layers):
         p = f"l{i}."
         norm_tensors(p + "norm1")
         if l.has_ff:
             norm_tensors(p + "norm2")
+        if cfg.design.hyper:
+            for q in ("hc1.", "hc2.") if l.has_ff else ("hc1.",):
+                out[p + q + "in"], out[p + q + "out"], out[p + q + "mix"] = (cfg.streams,), (cfg.streams,), (cfg.streams, cfg.streams)
         m = p + "mix."
-        if l.type == "attention" and l.values_are_keys:
+        if l.type == "attention" and l.talk:
+            out[m + "q"], out[m + "q.b"] = (l.heads * l.dim, d), (l.heads * l.dim,)
+            out[m + "k"], out[m + "k.b"] = (l.kv_heads * l.dim, d), (l.kv_heads * l.dim,)
+            out[m + "v"], out[m + "v.b"] = (l.kv_heads * l.vdim, d), (l.kv_heads * l.vdim,)
+            out[m + "talk"], out[m + "o"] = (l.heads, l.heads), (d, l.heads * l.vdim)
+        elif l.type == "latent_attention" and l.gate_full:
+            out[m + "q"] = (l.heads * (l.dim + l.rot_dim), d)
+            if l.owns_latent:
+                out[m + "dkv"], out[m + "dkv.norm"] = (l.kv_rank + l.rot_dim, d), (l.kv_rank,)
+            out[m + "uk"], out[m + "uv"] = (l.heads * l.dim, l.kv_rank), (l.heads * l.vdim, l.kv_rank)
+            out[m + "g"], out[m + "o"] = (l.heads * l.vdim, d), (d, l.heads * l.vdim)
+        elif l.type == "attention" and l.values_are_keys:
             out[m + "q"], out[m + "k"] = (l.heads * l.dim, d), (l.kv_heads * l.dim, d)
             out[m + "o"] = (d, l.heads * l.vdim)
         elif l.type == "attention":
@@ -537,6 +637,8 @@ def param_shapes(cfg: HybridConfig) -> Dict[str, tuple]:
             if cfg.design.dense_ff == "glu_relu":
                 out[f + "gate"] = (l.ff, d)
             out[f + "up"], out[f + "down"] = (l.ff, d), (d, l.ff)
+            if cfg.design.dense_ff == "xielu":
+                out[f + "up.b"], out[f + "down.b"], out[f + "act"] = (l.ff,), (d,), (2,)
     norm_tensors("final.norm")
     if not cfg.design.tied_head:
         out["head"] = (cfg.vocab_size, d)
@@ -556,9 +658,9 @@ class StepLayout:
 
 class HybridCache:
     """Paged keys / values of the attention layers that own any, the paged compressed rows of the
-    latent-attention layers, and the fp32 state slots of the recurrent layers, in ONE pool. Key
+    latent-attention layers that own any, and the fp32 state slots of the recurrent layers, in ONE pool. Key
     planes are [blocks, G, BS, dim], value planes [blocks, G, BS, vdim], latent planes
-    [blocks, 1, BS, kv_rank] (keys and values at once) in the model's activation type; a state
+    [blocks, 1, BS, kv_rank + rot_dim] (keys; their first kv_rank columns are the values) in the model's activation type; a state
     plane is [slots, size] fp32. Planes belong to layer RUNS (``HybridConfig.runs``): a layer that a
     loop runs several times has a set per pass; without a loop run r is layer r."""
 
@@ -579,8 +681,8 @@ class HybridCache:
                 plan.append(("k", i, take(num_blocks * l.kv_heads * block_size * l.dim * es)))
                 if not (l.values_are_keys and l.rot_dims == 0):      # (un-rotated keys that are the values: one plane)
                     plan.append(("v", i, take(num_blocks * l.kv_heads * block_size * l.vdim * es)))
-            elif l.type == "latent_attention":
-                plan.append(("c", i, take(num_blocks * block_size * l.kv_rank * es)))
+            elif l.owns_latent:
+                plan.append(("c", i, take(num_blocks * block_size * (l.kv_rank + l.rot_dim) * es)))
             elif l.state_size():
                 plan.append(("s", i, take(max(1, num_slots) * l.state_size() * 4)))
         total = max(off, 256)
@@ -604,8 +706,10 @@ class HybridCache:
                 n = num_blocks * l.kv_heads * block_size * l.vdim * es
                 self._v[i] = raw[at:at + n].view(dtype).view(num_blocks, l.kv_heads, block_size, l.vdim)
             elif kind == "c":
-                n = num_blocks * block_size * l.kv_rank * es
-                self._k[i] = self._v[i] = raw[at:at + n].view(dtype).view(num_blocks, 1, block_size, l.kv_rank)
+                w = l.kv_rank + l.rot_dim
+                n = num_blocks * block_size * w * es
+                self._k[i] = raw[at:at + n].view(dtype).view(num_blocks, 1, block_size, w)
+                self._v[i] = self._k[i][..., :l.kv_rank]     # (the compressed row: the first columns of the same rows)
             else:
                 n = max(1, num_slots) * l.state_size() * 4
                 self._s[i] = raw[at:at + n].view(torch.float32).view(max(1, num_slots), l.state_size())
@@ -662,6 +766,21 @@ class HybridLayer:
     experts_down: object = None                     # [E, d, ff]
     shared_up: Optional[ops.LinearWeight] = None
     shared_down: Optional[ops.LinearWeight] = None
+    inv_freq_v: Optional[torch.Tensor] = None       # attention whose values turn: fp64 [vdim/2]
+    talk: Optional[torch.Tensor] = None             # fp32 [H, H]: new head h's weights = sum_g talk[h, g] head g's
+    act: Optional[Tuple[float, float]] = None       # xIELU: (softplus(p), 1/2 + softplus(q))
+    hc1: Optional["StreamWeights"] = None           # parallel residual streams: the mixer's read / write weights
+    hc2: Optional["StreamWeights"] = None           # the feed-forward's
+
+
+@dataclass
+class StreamWeights:
+    """How one sublayer reads S parallel residual streams (``read`` [S]) and writes them (``mix`` [S, S] from -> to,
+    ``write`` [S] shares of its result), fp32."""
+
+    read: torch.Tensor
+    write: torch.Tensor
+    mix: torch.Tensor
 
 
 class HybridModel:
@@ -682,6 +801,8 @@ class HybridModel:
         self.final_norm: Optional[torch.Tensor] = None
         self.lm_head: Optional[ops.LinearWeight] = None
         self.loop_in: Optional[ops.LinearWeight] = None     # [d, 2 d]: the stream's re-injection before every pass of a loop
+        self.embed_norm: Optional[torch.Tensor] = None      # fp32 [d]: norm weight on the embedding rows
+        self.stream_sum: Optional[torch.Tensor] = None      # fp32 [S] of ones: the model's output reads every stream once
         self.layers: List[HybridLayer] = []
         self._rows: Dict[int, Tuple[torch.Tensor, torch.Tensor]] = {}
         self._max_len = 1
@@ -731,11 +852,39 @@ class HybridModel:
         # (a tied head is the embedding table once more, in the layout of the matrix products)
         self.lm_head = lin(load("embed" if c.design.tied_head else "head"))
         self.loop_in = lin(load("loop.in")) if c.looped else None
+        self.embed_norm = f32(load("embed.norm")) if c.design.embed_norm else None
+        self.stream_sum = torch.ones(c.streams, dtype=torch.float32, device=dev) if c.design.hyper else None
+
+        def inv_freqs(base: float, dims: int) -> torch.Tensor:
+            return torch.tensor([base ** (-2.0 * j / dims) for j in range(dims // 2)], dtype=torch.float64).to(dev)
         self.layers = []
         for i, l in enumerate(c.layers):
             p, m = f"l{i}.", f"l{i}.mix."
             kw = {}
-            if l.type == "attention" and l.values_are_keys:
+            if c.design.hyper:
+                for q in ("hc1", "hc2") if l.has_ff else ("hc1",):
+                    kw[q] = StreamWeights(f32(load(p + q + ".in")), f32(load(p + q + ".out")), f32(load(p + q + ".mix")))
+            if l.type == "attention" and l.talk:
+                if l.rot_dims:
+                    kw["inv_freq"] = inv_freqs(l.rot_base, l.rot_dims)
+                if l.rotate_values:
+                    kw["inv_freq_v"] = inv_freqs(l.rot_base, l.vdim)
+                kw["talk"] = f32(load(m + "talk"))
+                proj = lin(torch.cat([load(m + n) for n in ("q", "k", "v")], 0),
+                           torch.cat([load(m + n + ".b") for n in ("q", "k", "v")], 0), pad=True)
+                out = lin(load(m + "o"))
+            elif l.type == "latent_attention" and l.gate_full:
+                # queries (head by head: plain | turned part) | compressed row | shared key part | a gate logit per output
+                names = ("q", "dkv", "g") if l.owns_latent else ("q", "g")
+                proj = lin(torch.cat([load(m + n) for n in names], 0), pad=True)
+                if l.owns_latent:
+                    kw["latent_norm"] = f32(load(m + "dkv.norm"))
+                if l.rot_dim:
+                    kw["inv_freq"] = inv_freqs(l.rot_base, l.rot_dim)
+                kw["key_up_t"] = load(m + "uk").view(l.heads, l.dim, l.kv_rank).transpose(1, 2).to(dt).contiguous()
+                kw["value_up"] = load(m + "uv").view(l.heads, l.vdim, l.kv_rank).to(dt).contiguous()
+                out = lin(load(m + "o"))
+            elif l.type == "attention" and l.values_are_keys:
                 half = l.rot_dims // 2
                 if half:
                     kw["inv_freq"] = torch.tensor([l.rot_base ** (-2.0 * j / l.rot_dims) for j in range(half)],
@@ -815,6 +964,11 @@ class HybridModel:
                     kw["experts_down"] = ops.ExpertWeights.from_dense(downs, dev)
                 else:
                     kw["experts_up"], kw["experts_down"] = ups.to(dt).contiguous(), downs.to(dt).contiguous()
+            elif l.ff and c.design.dense_ff == "xielu":
+                a = load(f + "act").double().cpu()
+                sp = torch.nn.functional.softplus(a)
+                kw.update(up=lin(load(f + "up"), load(f + "up.b")), down=lin(load(f + "down"), load(f + "down.b")),
+                          act=(float(sp[0]), 0.5 + float(sp[1])))
             elif l.ff:
                 if c.design.dense_ff == "glu_relu":
                     kw["gate_up"] = lin(torch.cat([load(f + "gate"), load(f + "up")], 0))
@@ -845,7 +999,13 @@ class HybridModel:
             gen.manual_seed((seed * 1000003 + zlib.crc32(name.encode())) & 0x7FFFFFFFFFFFFFFF)
             offset_norm = cfg.design.norm_offset != 0.0 and name.split(".")[-1] in ("norm1", "norm2") or \
                 (cfg.design.norm_offset != 0.0 and name == "final.norm")
-            if name.endswith(".alpha"):
+            if ".hc" in name:                                    # streams that neither die out nor blow up
+                n = cfg.streams
+                t = {"in": torch.full(shape, 1.0 / n), "out": torch.ones(shape), "mix": torch.eye(n)}[name.split(".")[-1]]
+                t = t + 0.05 * torch.randn(shape, generator=gen)
+            elif name.endswith("mix.talk"):
+                t = torch.eye(shape[0]) + 0.1 * torch.randn(shape, generator=gen)
+            elif name.endswith(".alpha"):
                 t = 0.6 + 0.1 * torch.randn(shape, generator=gen)
             elif len(shape) == 2:
                 scale = cfg.hidden_size ** -0.5 if cfg.design.tied_head else 1.0     # (the table is the head too)
@@ -870,7 +1030,7 @@ class HybridModel:
         for L in self.layers:
             for w in (L.proj, L.out, L.up, L.down, L.decay_up, L.gate_up, L.router, L.shared_up, L.shared_down):
                 n += w.nbytes() if w is not None else 0
-            for t in (L.key_up_t, L.value_up, L.experts_up, L.experts_down):
+            for t in (L.key_up_t, L.value_up, L.experts_up, L.experts_down, L.talk):
                 t = t.data if isinstance(t, ops.ExpertWeights) else t
                 n += t.numel() * t.element_size() if t is not None else 0
         return n
@@ -912,6 +1072,8 @@ class HybridModel:
         T = token_ids.numel()
         self._portions = (meta.block_tables.shape[0], meta.prefill_tokens if meta.riders is not None else T) \
             if meta.is_prefill else (0, 0)
+        if c.design.hyper:
+            return self._forward_streams(token_ids, positions, slot_mapping, meta, lay, cache, taps)
         if c.design.pre_norm:
             return self._forward_pre_norm(token_ids, positions, slot_mapping, meta, lay, cache, taps)
         x, xa = ops.embed_rows(token_ids, self.embed, dt, meta.token_feed)
@@ -985,6 +1147,38 @@ class HybridModel:
                 taps.append(x.clone())
         return x
 
+    def _forward_streams(self, token_ids, positions, slot_mapping, meta, lay: StepLayout, cache: HybridCache,
+                         taps: Optional[list]) -> torch.Tensor:
+        """Layers around a residual of S parallel streams (fp32 [T, S, d]). One launch sits between two sublayers:
+        it writes the first one's result into the streams (every new stream a mixture of the old ones plus its
+        share), forms the second one's input from the new streams and norms it. The last launch of the step
+        returns the sum of the streams, which is what ``logits`` norms."""
+        c, dt, eps = self.cfg, self.dtype, self.cfg.rms_eps
+        x0, _ = ops.embed_rows(token_ids, self.embed, None, meta.token_feed)
+        xs = ops.hc_init(x0, self.embed_norm, eps, c.streams)
+        runs = c.runs
+        first = self.layers[runs[0][0]]
+        xa = ops.hc_step(xs, None, None, None, first.hc1.read, first.norm1, eps, dt)
+        x = None
+        for r, (i, _) in enumerate(runs):
+            L = self.layers[i]
+            l, hc = L.spec, L.hc1
+            if l.type == "latent_attention":
+                y = self._latent_attention_rot(r, L, xa, positions, slot_mapping, lay, cache)
+            else:
+                y = self._attention_talk(r, L, xa, positions, slot_mapping, lay, cache)
+            if l.has_ff:
+                xa = ops.hc_step(xs, y, hc.mix, hc.write, L.hc2.read, L.norm2, eps, dt)
+                y, hc = self._dense_ff(L, xa), L.hc2
+            if r + 1 == len(runs):
+                x = ops.hc_step(xs, y, hc.mix, hc.write, self.stream_sum, None, eps, None)
+            else:
+                nxt = self.layers[runs[r + 1][0]]
+                xa = ops.hc_step(xs, y, hc.mix, hc.write, nxt.hc1.read, nxt.norm1, eps, dt)
+            if taps is not None:
+                taps.append(x.clone() if x is not None else ops.hc_step(xs, None, None, None, self.stream_sum, None, eps, None))
+        return x
+
     def _residual_norm(self, x: torch.Tensor, y: Optional[torch.Tensor], norm, out: Optional[torch.Tensor] = None):
         """x += m * y (when y is given) and the design's norm of the new x in the activation type (when a
         norm is given; with ``out`` and no norm: the stream itself, cast, into that column block)."""
@@ -999,6 +1193,8 @@ class HybridModel:
         return xa
 
     def _dense_ff(self, L: HybridLayer, xa: torch.Tensor) -> torch.Tensor:
+        if L.act is not None:               # (biases ride in the products)
+            return ops.linear(ops.xielu(ops.linear(xa, L.up, out_f32=True), L.act[0], L.act[1], self.dtype), L.down, out_f32=True)
         if L.gate_up is not None:
             return ops.linear(ops.glu(ops.linear(xa, L.gate_up, out_f32=True), self.dtype, "relu"), L.down, out_f32=True)
         return ops.linear(self._relu2_up(xa, L.up), L.down, out_f32=True)
@@ -1057,6 +1253,43 @@ class HybridModel:
                             l.vdim, l.scale, 0, l.window, self.dtype, n_portions=self._portions[0],
                             portion_rows=self._portions[1], max_len=self._max_len)
         return ops.linear(a, L.out, out_f32=True)
+
+    def _attention_talk(self, r: int, L: HybridLayer, xa, positions, slot_mapping, lay: StepLayout, cache: HybridCache):
+        """Attention whose heads' softmax weights are mixed before they meet the values. The mix is linear in the
+        weights, so it is applied behind the weighted sums: the attention kernels give every head's weights on the
+        values of EVERY key/value head (fp32), and one launch mixes those sums per head and turns the result back
+        by the row's position (the values were cached turned by their own)."""
+        l = L.spec
+        kc, vc = cache.k(r), cache.v(r)
+        qkv = ops.linear(xa, L.proj, out_f32=True)
+        q = ops.rope_qkv_write(qkv, L.inv_freq, L.inv_freq_v, positions, slot_mapping, kc, vc, l.heads, l.kv_heads, l.dim,
+                               l.vdim, l.rot_dims)
+        o = ops.attn_masked(q, kc, vc, lay.block_tables, lay.cu_q, lay.row_seq, positions, l.heads, l.kv_heads, l.dim, l.vdim,
+                            l.scale, 0, l.window, torch.float32, n_portions=self._portions[0], portion_rows=self._portions[1],
+                            max_len=self._max_len, softcap=l.softcap, sink=l.sink, all_value_heads=True)
+        a = ops.talk_mix(o, L.talk, positions, L.inv_freq_v, l.heads, l.kv_heads, l.vdim, self.dtype)
+        return ops.linear(a, L.out, out_f32=True)
+
+    def _latent_attention_rot(self, r: int, L: HybridLayer, xa, positions, slot_mapping, lay: StepLayout, cache: HybridCache):
+        """Latent attention with a turned key part shared by all heads. The cached row is [compressed row | key part];
+        the query of head h in the same coordinates is [U_h^T q_plain | turned q part], so that one dot product with
+        the cached row is the head's score; the values are the first kv_rank columns of the same rows."""
+        l = L.spec
+        H, D, rd, R, Dv = l.heads, l.dim, l.rot_dim, l.kv_rank, l.vdim
+        nq, W = H * (D + rd), R + rd
+        own = l.owns_latent
+        cc = cache.k(r if own else l.kv_from)
+        proj = ops.linear(xa, L.proj, out_f32=True)                 # q | (compressed row | key part) | gate logits
+        qlat = torch.empty(proj.shape[0], H * W, dtype=torch.float32, device=proj.device)
+        ops.latent_rope_write(proj, nq, L.latent_norm, self.cfg.rms_eps, L.inv_freq, positions, slot_mapping,
+                              cc if own else None, qlat, H, D, R, rd)
+        ops.head_linear(proj, L.key_up_t, torch.float32, x_head_stride=D + rd, out=qlat, out_head_stride=W)
+        a = ops.attn_masked(qlat, cc, cc[..., :R], lay.block_tables, lay.cu_q, lay.row_seq, positions, H, 1, W, R, l.scale,
+                            0, l.window, torch.float32, n_portions=self._portions[0], portion_rows=self._portions[1],
+                            max_len=self._max_len)
+        g0 = nq + (W if own else 0)
+        o = ops.head_linear(a, L.value_up, self.dtype, gate=proj[:, g0:g0 + H * Dv], gate_full=True)
+        return ops.linear(o, L.out, out_f32=True)
 
     def _latent_attention(self, i: int, L: HybridLayer, xa, positions, slot_mapping, lay: StepLayout, cache: HybridCache):
         l = L.spec

@@ -24,7 +24,7 @@ class Family:
 
 # the designs models/hybrid.py serves (its ``DESIGNS``), named here so that finding a checkpoint's
 # family does not import the model code
-HYBRID_DESIGNS = ("Nidozen", "Telurax", "Surevik")
+HYBRID_DESIGNS = ("Nidozen", "Telurax", "Surevik", "Gizilorn")
 
 _FAMILIES: Dict[str, Family] = {}
 _BY_KEY: Dict[Tuple[str, str], str] = {}          # (config key, value) -> family name

@@ -1068,14 +1068,29 @@ def attn_tile_ok(D: int, Dv: int) -> bool:
 ATTN_TILE_MIN_ROWS = int(os.environ.get("LC_ATTN_TILE_MIN_ROWS", "16"))
 
 
+def _cache_ld(c: torch.Tensor, G: int, width: int, what: str) -> int:
+    """Row stride of a cache plane [blocks, G, BS, width] that may be a column block of wider rows."""
+    BS, ld = c.shape[2], c.stride(2)
+    if c.dim() != 4 or c.shape[1] != G or c.shape[3] != width or c.stride(3) != 1 or ld < width or \
+            c.stride(1) != BS * ld or c.stride(0) != G * BS * ld:
+        raise ValueError(f"attn_masked: the {what} plane does not fit the head sizes")
+    return ld
+
+
 def attn_masked(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_tables: torch.Tensor,
                 cu_q: torch.Tensor, row_seq: torch.Tensor, positions: torch.Tensor, H: int, G: int, D: int, Dv: int,
                 scale: float, chunk: int, window: int, act_dtype: torch.dtype, n_portions: int = 0,
-                portion_rows: int = 0, max_len: int = 0) -> torch.Tensor:
+                portion_rows: int = 0, max_len: int = 0, softcap: float = 0.0, sink: bool = False,
+                all_value_heads: bool = False) -> torch.Tensor:
     """Attention of fp32 queries [T, H*D] over paged keys / values of widths D / Dv. The row at
     position p sees keys j <= p with j >= floor(p / chunk) * chunk (``chunk`` > 0) and
     j > p - window (``window`` > 0), counted from the start of its sequence. ``row_seq`` [T]
     names each row's sequence (row of ``block_tables``); scores, weights and sums are fp32.
+    The planes are [blocks, G, BS, D] / [blocks, G, BS, Dv] and may be column blocks of wider rows
+    (a latent row that is key and value at once). ``softcap`` > 0: the scaled score s becomes
+    softcap * tanh(s / softcap). ``sink``: the softmax has a silent extra entry of score 0, so the
+    weights sum to less than one. ``all_value_heads``: every query head's weights are applied to
+    the values of ALL G key/value heads; the result is [T, H * G * Dv] (head, value head, column).
 
     Two kernels: the first ``n_portions`` sequences (rows [0, portion_rows), the longest of
     ``max_len`` rows) are prompt portions and go, 64 rows of a head per block, through fp32 MFMA
@@ -1083,26 +1098,45 @@ def attn_masked(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, b
     through the row kernel, one wave per (row, head)."""
     if not q.is_cuda:
         return ref.attn_masked(q, k_cache, v_cache, block_tables, cu_q, positions, H, G, D, Dv, scale, chunk, window,
-                               act_dtype)
+                               act_dtype, softcap, sink, all_value_heads)
     T = q.shape[0]
     if q.dtype != torch.float32 or not q.is_contiguous() or k_cache.dtype != v_cache.dtype:
         raise ValueError("attn_masked: contiguous fp32 queries, caches of one type")
-    if k_cache.shape[1:] != (G, k_cache.shape[2], D) or v_cache.shape[1:] != (G, k_cache.shape[2], Dv):
-        raise ValueError("attn_masked: cache planes do not fit the head sizes")
+    k_ld, v_ld = _cache_ld(k_cache, G, D, "key"), _cache_ld(v_cache, G, Dv, "value")
+    if k_cache.shape[2] != v_cache.shape[2]:
+        raise ValueError("attn_masked: key and value planes of one block size")
     if not 0 <= portion_rows <= T or n_portions > block_tables.shape[0]:
         raise ValueError("attn_masked: the portions exceed the step")
-    out = torch.empty(T, H * Dv, dtype=act_dtype, device=q.device)
+    nv = G if all_value_heads else 1
+    o_ld = nv * Dv
+    out = torch.empty(T, H * o_ld, dtype=act_dtype, device=q.device)
     BS, MB, cf, af = k_cache.shape[2], block_tables.shape[1], _f32flag(k_cache.dtype), _f32flag(act_dtype)
+
+    def value_groups(cap: int):
+        """(first value head or -1, heads, first output column) per launch: as many value heads side by side as fit."""
+        if not all_value_heads:
+            return [(-1, 1, 0)] if Dv <= cap else []
+        n = cap // Dv
+        return [(v0, min(n, G - v0), v0 * Dv) for v0 in range(0, G, n)] if n else []
+    opts = (float(softcap), 1 if sink else 0)
     first = 0
-    if n_portions > 0 and portion_rows > 0 and max_len >= ATTN_TILE_MIN_ROWS and attn_tile_ok(D, Dv):
-        _hip().call("lc_attn_tile", q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), cf, block_tables.data_ptr(),
-                    MB, cu_q.data_ptr(), positions.data_ptr(), out.data_ptr(), af, int(n_portions), int(max_len), H, G,
-                    D, Dv, BS, float(scale), int(chunk), int(window))
+    tile_cols = max([n * Dv for n in range(1, nv + 1) if attn_tile_ok(D, n * Dv)] or [0])
+    aligned = k_ld % 8 == 0 and v_ld % 8 == 0 and k_cache.data_ptr() % 16 == 0 and v_cache.data_ptr() % 16 == 0
+    if n_portions > 0 and portion_rows > 0 and max_len >= ATTN_TILE_MIN_ROWS and tile_cols and aligned:
+        for vh0, nvh, col0 in value_groups(tile_cols):
+            _hip().call("lc_attn_tile", q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), cf, block_tables.data_ptr(),
+                        MB, cu_q.data_ptr(), positions.data_ptr(), out.data_ptr(), af, int(n_portions), int(max_len), H, G,
+                        D, Dv, BS, float(scale), int(chunk), int(window), k_ld, v_ld, *opts, vh0, nvh, o_ld, col0)
         first = portion_rows
     if first < T:
-        _hip().call("lc_attn_masked", q[first:].data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), cf,
-                    block_tables.data_ptr(), MB, row_seq[first:].data_ptr(), positions[first:].data_ptr(),
-                    out[first:].data_ptr(), af, T - first, H, G, D, Dv, BS, float(scale), int(chunk), int(window))
+        groups = value_groups(512)
+        if not groups:
+            raise ValueError("attn_masked: the row kernel takes value widths up to 512")
+        for vh0, nvh, col0 in groups:
+            _hip().call("lc_attn_masked", q[first:].data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), cf,
+                        block_tables.data_ptr(), MB, row_seq[first:].data_ptr(), positions[first:].data_ptr(),
+                        out[first:].data_ptr(), af, T - first, H, G, D, Dv, BS, float(scale), int(chunk), int(window),
+                        k_ld, v_ld, *opts, vh0, nvh, o_ld, col0)
     return out
 
 
@@ -1140,22 +1174,35 @@ def latent_write(proj: torch.Tensor, col0: int, w: torch.Tensor, eps: float, slo
                 slot_mapping.data_ptr(), cache.data_ptr(), _f32flag(cache.dtype), cache.shape[2], proj.shape[0])
 
 
-def head_linear(x: torch.Tensor, W: torch.Tensor, out_dtype: torch.dtype, gate: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """Per-head products y[t, h] = W[h] x[t, h]: x [T, H*K] (may be a column slice), W [H, N, K]
+def head_linear(x: torch.Tensor, W: torch.Tensor, out_dtype: torch.dtype, gate: Optional[torch.Tensor] = None,
+                x_head_stride: Optional[int] = None, out: Optional[torch.Tensor] = None,
+                out_head_stride: Optional[int] = None, gate_full: bool = False) -> torch.Tensor:
+    """Per-head products y[t, h] = W[h] x[t, h]: x [T, >= H*K] (may be a column slice), W [H, N, K]
     row-major, y [T, H*N] in ``out_dtype``; fp32 accumulation. ``gate`` [T, H] (logits, may be a
-    column slice): y[t, h] *= sigmoid(gate[t, h])."""
-    if not x.is_cuda:
-        return ref.head_linear(x, W, out_dtype, gate)
+    column slice): y[t, h] *= sigmoid(gate[t, h]); with ``gate_full`` the gate is [T, H*N], a logit per
+    output. ``x_head_stride``: head h's inputs start at column h * x_head_stride (default K: heads side by
+    side). ``out`` / ``out_head_stride``: write head h's outputs from column h * out_head_stride of this
+    matrix instead of a new one (the other columns are left alone)."""
     H, N, K = W.shape
     M = x.shape[0]
-    if x.shape[1] != H * K or x.stride(1) != 1 or not W.is_contiguous():
+    xs = K if x_head_stride is None else int(x_head_stride)
+    os_ = N if out_head_stride is None else int(out_head_stride)
+    if xs < K or x.shape[1] < (H - 1) * xs + K or x.stride(1) != 1 or not W.is_contiguous():
         raise ValueError("head_linear: activations [T, H*K] against weights [H, N, K]")
-    if gate is not None and (gate.shape != (M, H) or gate.dtype != torch.float32 or gate.stride(1) != 1):
-        raise ValueError("head_linear: the gate is an fp32 [T, H] matrix")
-    y = torch.empty(M, H * N, dtype=out_dtype, device=x.device)
-    _hip().call("lc_head_linear", x.data_ptr(), _f32flag(x.dtype), max(x.stride(0), H * K), W.data_ptr(), _f32flag(W.dtype),
-                y.data_ptr(), _f32flag(out_dtype), _hip().ptr(gate), max(gate.stride(0), H) if gate is not None else 0,
-                M, H, N, K)
+    if gate is not None and (gate.shape != (M, H * N if gate_full else H) or gate.dtype != torch.float32 or gate.stride(1) != 1):
+        raise ValueError("head_linear: the gate is an fp32 [T, H] matrix ([T, H*N] when it is a logit per output)")
+    if gate is None and gate_full:
+        raise ValueError("head_linear: a gate per output needs the gate")
+    if out is not None and (out.shape[0] != M or out.dtype != out_dtype or out.stride(1) != 1 or os_ < N
+                            or out.shape[1] < (H - 1) * os_ + N):
+        raise ValueError("head_linear: the output matrix does not hold the heads' blocks")
+    if not x.is_cuda:
+        return ref.head_linear(x, W, out_dtype, gate, xs, out, os_, gate_full)
+    y = out if out is not None else torch.empty(M, (H - 1) * os_ + N, dtype=out_dtype, device=x.device)
+    _hip().call("lc_head_linear", x.data_ptr(), _f32flag(x.dtype), max(x.stride(0), (H - 1) * xs + K), W.data_ptr(),
+                _f32flag(W.dtype), y.data_ptr(), _f32flag(out_dtype), _hip().ptr(gate),
+                max(gate.stride(0), gate.shape[1]) if gate is not None else 0, M, H, N, K, xs,
+                max(y.stride(0), (H - 1) * os_ + N), os_, 1 if gate_full else 0)
     return y
 
 
@@ -1399,4 +1446,143 @@ def glu_clamped(y: torch.Tensor, col_gate: int, col_up: int, n: int, limit: floa
     _hip().call("lc_glu_clamped", y.data_ptr(), y.stride(0) if R > 1 else max(y.stride(0), y.shape[1]), int(col_gate),
                 int(col_up), int(n), float(limit), float(slope), float(shift), _hip().ptr(slot_of), _hip().ptr(wts),
                 out.data_ptr(), _f32flag(act_dtype), rows)
+    return out
+
+
+# ---- parallel residual streams, rotary values, mixed heads' weights, rotated latent keys, xIELU (hybrid_streams.hip) ----
+MAX_STREAMS = 8
+
+
+def hc_init(x0: torch.Tensor, w: torch.Tensor, eps: float, streams: int) -> torch.Tensor:
+    """The start of a residual of several parallel streams: fp32 [T, S, d], every stream the RMS norm of x0
+    (fp32 [T, d]) times w."""
+    T, d = x0.shape
+    if x0.dtype != torch.float32 or not x0.is_contiguous() or w.numel() != d or not 1 <= streams <= MAX_STREAMS:
+        raise ValueError(f"hc_init: a contiguous fp32 matrix, a weight per column, 1..{MAX_STREAMS} streams")
+    if not x0.is_cuda:
+        return ref.hc_init(x0, w, eps, streams)
+    xs = torch.empty(T, streams, d, dtype=torch.float32, device=x0.device)
+    _hip().call("lc_hc_init", x0.data_ptr(), w.data_ptr(), float(eps), xs.data_ptr(), T, streams, d)
+    return xs
+
+
+def hc_step(xs: torch.Tensor, y: Optional[torch.Tensor], mix: Optional[torch.Tensor], out_w: Optional[torch.Tensor],
+            in_w: Optional[torch.Tensor], norm_w: Optional[torch.Tensor], eps: float,
+            act_dtype: Optional[torch.dtype]) -> Optional[torch.Tensor]:
+    """One launch between two sublayers of a residual of S parallel streams xs (fp32 [T, S, d], in place). With
+    ``y`` (fp32 [T, d], the sublayer's result): every new stream is a mixture of the old ones plus its share of
+    y, xs[:, j] <- sum_s mix[s, j] xs[:, s] + out_w[j] y. With ``in_w``: the next sublayer's input
+    u = sum_s in_w[s] xs[:, s]; returned RMS-normed times ``norm_w`` in ``act_dtype``, or, without a norm weight,
+    as it is in fp32. Without ``in_w`` nothing is returned."""
+    T, S, d = xs.shape
+    if xs.dtype != torch.float32 or not xs.is_contiguous() or S > MAX_STREAMS:
+        raise ValueError(f"hc_step: the streams are a contiguous fp32 [T, S, d] tensor, S <= {MAX_STREAMS}")
+    if y is not None and (y.shape != (T, d) or y.dtype != torch.float32 or mix is None or out_w is None
+                          or mix.numel() != S * S or out_w.numel() != S):
+        raise ValueError("hc_step: an fp32 [T, d] result with mix [S, S] and out [S]")
+    if (in_w is not None and in_w.numel() != S) or (norm_w is not None and (in_w is None or norm_w.numel() != d)):
+        raise ValueError("hc_step: in [S], and a norm weight per column only with it")
+    for c in (mix, out_w, in_w, norm_w):
+        if c is not None and (c.dtype != torch.float32 or not c.is_contiguous()):
+            raise ValueError("hc_step: fp32 coefficients")
+    if not xs.is_cuda:
+        return ref.hc_step(xs, y, mix, out_w, in_w, norm_w, eps, act_dtype)
+    if y is None and in_w is None:
+        return None
+    u = torch.empty(T, d, dtype=torch.float32, device=xs.device) if in_w is not None and norm_w is None else None
+    xa = torch.empty(T, d, dtype=act_dtype, device=xs.device) if norm_w is not None else None
+    _hip().call("lc_hc_step", xs.data_ptr(), _hip().ptr(y.contiguous() if y is not None else None), _hip().ptr(mix),
+                _hip().ptr(out_w), _hip().ptr(in_w), _hip().ptr(norm_w), float(eps), _hip().ptr(u), _hip().ptr(xa),
+                _f32flag(act_dtype) if xa is not None else 0, T, S, d)
+    return xa if xa is not None else u
+
+
+def rope_qkv_write(qkv: torch.Tensor, inv_freq: Optional[torch.Tensor], inv_freq_v: Optional[torch.Tensor],
+                   positions: torch.Tensor, slot_mapping: torch.Tensor, k_cache: Optional[torch.Tensor],
+                   v_cache: Optional[torch.Tensor], H: int, G: int, D: int, Dv: int, rot_dims: int, pairs: bool = False,
+                   v_pairs: bool = False) -> torch.Tensor:
+    """Rotary positions and the paged cache write of an attention layer with a value projection: qkv fp32
+    [T, >= H D + G (D + Dv)] = q | k | v. The first ``rot_dims`` coordinates of every query and key head turn by
+    position * inv_freq[i] (fp64 [rot_dims / 2]); ``pairs``: neighbours (2i, 2i + 1) turn together, otherwise i
+    with i + rot_dims / 2. With ``inv_freq_v`` (fp64 [Dv / 2]) every value head turns over its whole width by its
+    own position (layout ``v_pairs``) and is cached so. Keys go to ``k_cache`` [blocks, G, BS, D], values to
+    ``v_cache`` [blocks, G, BS, Dv]. Returns the turned q fp32 [T, H*D]."""
+    if rot_dims and (inv_freq is None or inv_freq.dtype != torch.float64 or inv_freq.numel() != rot_dims // 2):
+        raise ValueError("rope_qkv_write: rot_dims / 2 fp64 frequencies are needed")
+    if inv_freq_v is not None and (inv_freq_v.dtype != torch.float64 or inv_freq_v.numel() * 2 != Dv):
+        raise ValueError("rope_qkv_write: Dv / 2 fp64 frequencies for the values")
+    if k_cache is not None and (k_cache.shape[1:] != (G, k_cache.shape[2], D) or v_cache.shape[1:] != (G, k_cache.shape[2], Dv)
+                                or not k_cache.is_contiguous() or not v_cache.is_contiguous() or k_cache.dtype != v_cache.dtype):
+        raise ValueError("rope_qkv_write: cache planes do not fit the head sizes")
+    if qkv.dtype != torch.float32 or qkv.stride(1) != 1 or qkv.shape[1] < H * D + G * (D + Dv):
+        raise ValueError("rope_qkv_write: fp32 projections q | k | v")
+    if not qkv.is_cuda:
+        return ref.rope_qkv_write(qkv, inv_freq, inv_freq_v, positions, slot_mapping, k_cache, v_cache, H, G, D, Dv,
+                                  rot_dims, pairs, v_pairs)
+    T = qkv.shape[0]
+    q = torch.empty(T, H * D, dtype=torch.float32, device=qkv.device)
+    _hip().call("lc_rope_qkv_write", qkv.data_ptr(), max(qkv.stride(0), qkv.shape[1]), _hip().ptr(inv_freq),
+                _hip().ptr(inv_freq_v), positions.data_ptr(), slot_mapping.data_ptr(), _hip().ptr(k_cache), _hip().ptr(v_cache),
+                _f32flag(k_cache.dtype) if k_cache is not None else 0, q.data_ptr(), T, H, G, D, Dv,
+                k_cache.shape[2] if k_cache is not None else 1, rot_dims, 1 if pairs else 0, 1 if v_pairs else 0)
+    return q
+
+
+def talk_mix(o: torch.Tensor, talk: torch.Tensor, positions: torch.Tensor, inv_freq_v: Optional[torch.Tensor], H: int,
+             G: int, Dv: int, act_dtype: torch.dtype, v_pairs: bool = False) -> torch.Tensor:
+    """The heads' softmax weights mixed by ``talk`` (fp32 [H, H]: new head h = sum_g talk[h, g] head g), applied
+    behind the weighted sums: o fp32 [T, H * G * Dv] holds every head's weights on every value head
+    (``attn_masked(..., all_value_heads=True)``); out[t, h] = sum_g talk[h, g] o[t, g, h / (H / G)]. With
+    ``inv_freq_v`` (fp64 [Dv / 2]) each head's result turns back by its row's position over its whole width.
+    Returns [T, H * Dv] in ``act_dtype``."""
+    T = o.shape[0]
+    if o.dtype != torch.float32 or not o.is_contiguous() or o.shape[1] != H * G * Dv or talk.numel() != H * H or \
+            talk.dtype != torch.float32 or not talk.is_contiguous() or H % G:
+        raise ValueError("talk_mix: fp32 sums [T, H * G * Dv] and an fp32 [H, H] mixing matrix")
+    if inv_freq_v is not None and (inv_freq_v.dtype != torch.float64 or inv_freq_v.numel() * 2 != Dv):
+        raise ValueError("talk_mix: Dv / 2 fp64 frequencies")
+    if not o.is_cuda:
+        return ref.talk_mix(o, talk, positions, inv_freq_v, H, G, Dv, act_dtype, v_pairs)
+    out = torch.empty(T, H * Dv, dtype=act_dtype, device=o.device)
+    _hip().call("lc_talk_mix", o.data_ptr(), talk.data_ptr(), positions.data_ptr(), _hip().ptr(inv_freq_v), out.data_ptr(),
+                _f32flag(act_dtype), T, H, G, Dv, 1 if v_pairs else 0)
+    return out
+
+
+def latent_rope_write(proj: torch.Tensor, col_c: int, w: Optional[torch.Tensor], eps: float, inv_freq: Optional[torch.Tensor],
+                      positions: torch.Tensor, slot_mapping: torch.Tensor, cache: Optional[torch.Tensor], qlat: torch.Tensor,
+                      H: int, D: int, R: int, rd: int, pairs: bool = True) -> None:
+    """Latent attention whose cached row carries a rotated key part that all heads share. proj fp32 [T, ...]:
+    queries from column 0, head by head [D plain | rd to turn]; with ``cache`` ([blocks, 1, BS, R + rd]) also the
+    compressed row and the shared key part, R + rd columns from ``col_c`` on: the cache row at the token's slot
+    becomes rms_norm(compressed) * w | turned key part. The turned query parts go to columns R .. R + rd - 1 of each
+    head's block of ``qlat`` (fp32 [T, H * (R + rd)]). ``inv_freq`` fp64 [rd / 2]; ``pairs``: neighbours turn together."""
+    T = proj.shape[0]
+    if proj.dtype != torch.float32 or proj.stride(1) != 1 or proj.shape[1] < H * (D + rd):
+        raise ValueError("latent_rope_write: fp32 projections")
+    if qlat.shape != (T, H * (R + rd)) or qlat.dtype != torch.float32 or not qlat.is_contiguous():
+        raise ValueError("latent_rope_write: queries in the cached row's coordinates are fp32 [T, H * (R + rd)]")
+    if rd and (rd % 2 or inv_freq is None or inv_freq.dtype != torch.float64 or inv_freq.numel() != rd // 2):
+        raise ValueError("latent_rope_write: rd / 2 fp64 frequencies are needed")
+    if cache is not None and (cache.shape[1] != 1 or cache.shape[3] != R + rd or not cache.is_contiguous() or w is None
+                              or w.numel() != R or col_c < H * (D + rd) or col_c + R + rd > proj.shape[1]):
+        raise ValueError("latent_rope_write: a one-head cache plane of width R + rd and the compressed row's columns")
+    if not proj.is_cuda:
+        return ref.latent_rope_write(proj, col_c, w, eps, inv_freq, positions, slot_mapping, cache, qlat, H, D, R, rd, pairs)
+    _hip().call("lc_latent_rope_write", proj.data_ptr(), max(proj.stride(0), proj.shape[1]), int(col_c), _hip().ptr(w),
+                float(eps), _hip().ptr(inv_freq), positions.data_ptr(), slot_mapping.data_ptr(), _hip().ptr(cache),
+                _f32flag(cache.dtype) if cache is not None else 0, qlat.data_ptr(), T, H, D, R, rd,
+                cache.shape[2] if cache is not None else 1, 1 if pairs else 0)
+
+
+def xielu(y: torch.Tensor, ap: float, an: float, act_dtype: torch.dtype) -> torch.Tensor:
+    """xIELU of an fp32 matrix (may be a column slice): ap z^2 + z / 2 above zero, an (exp(z) - 1 - z) + z / 2 at
+    and below it, in ``act_dtype``."""
+    if not y.is_cuda:
+        return ref.xielu(y, ap, an, act_dtype)
+    if y.dim() != 2 or y.stride(1) != 1 or y.dtype != torch.float32:
+        raise ValueError("xielu: an fp32 matrix with unit column stride")
+    T, n = y.shape
+    out = torch.empty(T, n, dtype=act_dtype, device=y.device)
+    _hip().call("lc_xielu", y.data_ptr(), max(y.stride(0), n), out.data_ptr(), _f32flag(act_dtype), T, n, float(ap), float(an))
     return out

@@ -67,17 +67,26 @@ _SIGNATURES = {
     "lc_gla_scan": [_P, _I, _P, _P, _L, _P, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _P, _P, _P],
     "lc_headnorm_gate": [_P, _P, _P, _I, _P, _I, _I, _I, _I, _F, _I, _I, _I, _P, _P],
     "lc_qkv_prep": [_P, _I, _P, _P, _P, _P, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _F, _I, _P],
-    "lc_attn_masked": [_P, _P, _P, _I, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _I, _I, _P],
-    "lc_attn_tile": [_P, _P, _P, _I, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _F, _I, _I, _P],
+    "lc_attn_masked": [_P, _P, _P, _I, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _I, _I,
+                       _I, _I, _F, _I, _I, _I, _I, _I, _P],
+    "lc_attn_tile": [_P, _P, _P, _I, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _F, _I, _I,
+                     _I, _I, _F, _I, _I, _I, _I, _I, _P],
     "lc_gemm_any": [_P, _I, _I, _P, _I, _P, _P, _I, _I, _I, _I, _I, _P],
     "lc_add_rmsnorm": [_P, _P, _P, _F, _P, _I, _I, _I, _P],
     "lc_latent_write": [_P, _I, _I, _I, _P, _F, _P, _P, _I, _I, _I, _P],
-    "lc_head_linear": [_P, _I, _I, _P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _P],
+    "lc_head_linear": [_P, _I, _I, _P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P],
     "lc_mlstm_scan": [_P, _I, _P, _L, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _P, _P, _P],
     "lc_glu": [_P, _P, _I, _I, _I, _I, _P],
     "lc_add_dyt": [_P, _P, _F, _F, _P, _P, _P, _I, _I, _I, _I, _P],
     "lc_glu_clamped": [_P, _I, _I, _I, _I, _F, _F, _F, _P, _P, _P, _I, _I, _P],
     "lc_rope_pairs_write": [_P, _I, _P, _P, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _P],
+    # parallel residual streams, rotary values, mixed heads' weights, rotated latent keys, xIELU (hybrid_streams.hip)
+    "lc_hc_init": [_P, _P, _F, _P, _I, _I, _I, _P],
+    "lc_hc_step": [_P, _P, _P, _P, _P, _P, _F, _P, _P, _I, _I, _I, _I, _P],
+    "lc_rope_qkv_write": [_P, _I, _P, _P, _P, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P],
+    "lc_talk_mix": [_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P],
+    "lc_latent_rope_write": [_P, _I, _I, _P, _F, _P, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _P],
+    "lc_xielu": [_P, _I, _P, _I, _I, _I, _F, _F, _P],
     # routed feed-forwards of hybrid decoders (hybrid_moe.hip)
     "lc_route_grouped": [_P, _I, _P, _I, _I, _I, _I, _I, _F, _I, _P, _P, _P],
     "lc_moe_sort": [_P, _I, _I, _I, _P, _P, _P, _P, _P, _P],

@@ -400,12 +400,17 @@ def qkv_prep(qkv: torch.Tensor, q_norm: torch.Tensor, k_norm: Optional[torch.Ten
 
 
 def attn_masked(q: torch.Tensor, k_cache, v_cache, block_tables, cu_q, positions, H: int, G: int, D: int, Dv: int,
-                scale: float, chunk: int, window: int, act_dtype) -> torch.Tensor:
+                scale: float, chunk: int, window: int, act_dtype, softcap: float = 0.0, sink: bool = False,
+                all_value_heads: bool = False) -> torch.Tensor:
     """q fp32 [T, H*D]; paged keys [blocks, G, BS, D] and values [blocks, G, BS, Dv]. The row at
     position p sees keys j <= p with j >= floor(p / chunk) * chunk (``chunk`` > 0) and
-    j > p - window (``window`` > 0). Scores, softmax and the weighted sum in fp32."""
+    j > p - window (``window`` > 0). Scores, softmax and the weighted sum in fp32. ``softcap`` > 0: scores
+    become softcap * tanh(score / softcap); ``sink``: one is added to the softmax's denominator (an entry of
+    score 0 without a value); ``all_value_heads``: every head's weights meet the values of all G value heads,
+    result [T, H * G * Dv]."""
     T = q.shape[0]
-    out = torch.zeros(T, H * Dv, dtype=torch.float32, device=q.device)
+    nv = G if all_value_heads else 1
+    out = torch.zeros(T, H * nv * Dv, dtype=torch.float32, device=q.device)
     BS = k_cache.shape[2]
     rep = H // G
     for b in range(len(cu_q) - 1):
@@ -420,6 +425,8 @@ def attn_masked(q: torch.Tensor, k_cache, v_cache, block_tables, cu_q, positions
         V = v_cache[blocks].permute(1, 0, 2, 3).reshape(G, nb * BS, Dv)[:, :n].float()
         Q = q[r0:r1].float().view(r1 - r0, G, rep, D)
         sc = torch.einsum("qgrd,gkd->grqk", Q, K) * scale
+        if softcap > 0:
+            sc = softcap * torch.tanh(sc / softcap)
         key = torch.arange(n, device=q.device)[None, :]
         mask = key <= pos[:, None]
         if chunk > 0:
@@ -427,8 +434,16 @@ def attn_masked(q: torch.Tensor, k_cache, v_cache, block_tables, cu_q, positions
         if window > 0:
             mask &= key > pos[:, None] - window
         sc = sc.masked_fill(~mask[None, None], float("-inf"))
-        o = torch.einsum("grqk,gkv->qgrv", torch.softmax(sc, dim=-1), V)
-        out[r0:r1] = o.reshape(r1 - r0, H * Dv)
+        if sink:
+            m = sc.max(-1, keepdim=True).values.clamp_min(0.0)
+            e = torch.exp(sc - m)
+            w = e / (torch.exp(-m) + e.sum(-1, keepdim=True))
+        else:
+            w = torch.softmax(sc, dim=-1)
+        if all_value_heads:
+            out[r0:r1] = torch.einsum("grqk,ckv->qgrcv", w, V).reshape(r1 - r0, H * G * Dv)
+        else:
+            out[r0:r1] = torch.einsum("grqk,gkv->qgrv", w, V).reshape(r1 - r0, H * Dv)
     return out.to(act_dtype)
 
 
@@ -459,13 +474,25 @@ def latent_write(proj: torch.Tensor, col0: int, w: torch.Tensor, eps: float, slo
     cache[slots[ok] // BS, 0, slots[ok] % BS, :] = c[ok].to(cache.dtype)
 
 
-def head_linear(x: torch.Tensor, W: torch.Tensor, out_dtype, gate: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """x [T, H*K], W [H, N, K] -> y [T, H*N] with y[t, h] = W[h] x[t, h]; ``gate`` [T, H]: y[t, h] *= sigmoid(gate[t, h])."""
+def head_linear(x: torch.Tensor, W: torch.Tensor, out_dtype, gate: Optional[torch.Tensor] = None,
+                x_head_stride: Optional[int] = None, out: Optional[torch.Tensor] = None,
+                out_head_stride: Optional[int] = None, gate_full: bool = False) -> torch.Tensor:
+    """x [T, >= H*K], W [H, N, K] -> y with y[t, h] = W[h] x[t, h]; head h reads from column h * x_head_stride and
+    writes from column h * out_head_stride (of ``out`` when given); ``gate`` [T, H]: y[t, h] *= sigmoid(gate[t, h]),
+    or a logit per output, [T, H*N], with ``gate_full``."""
     H, N, K = W.shape
-    y = torch.einsum("thk,hnk->thn", x.float().reshape(x.shape[0], H, K), W.float())
+    T = x.shape[0]
+    xs = K if x_head_stride is None else x_head_stride
+    os_ = N if out_head_stride is None else out_head_stride
+    xh = torch.stack([x[:, h * xs:h * xs + K].float() for h in range(H)], 1)
+    y = torch.einsum("thk,hnk->thn", xh, W.float())
     if gate is not None:
-        y = y * torch.sigmoid(gate.float())[:, :, None]
-    return y.reshape(x.shape[0], H * N).to(out_dtype)
+        y = y * (torch.sigmoid(gate.float()).view(T, H, N) if gate_full else torch.sigmoid(gate.float())[:, :, None])
+    if out is None:
+        out = torch.zeros(T, (H - 1) * os_ + N, dtype=out_dtype, device=x.device)
+    for h in range(H):
+        out[:, h * os_:h * os_ + N] = y[:, h].to(out_dtype)
+    return out
 
 
 def capped(x: torch.Tensor, cap: float) -> torch.Tensor:
@@ -627,3 +654,99 @@ def glu_clamped(y: torch.Tensor, col_gate: int, col_up: int, n: int, limit: floa
         s[slot_of.long().reshape(-1)[:rows], 0] = wts.float().reshape(-1)[:rows] if wts is not None else 1.0
     g, u = torch.clamp(g * s, max=limit), torch.clamp(u * s, -limit, limit)
     return (g * torch.sigmoid(slope * g) * (u + shift)).to(act_dtype)
+
+
+# ------------------------------------------------------------------ hybrid decoders: parallel residual streams, rotary
+# values, mixed heads' weights, rotated latent keys, xIELU
+def hc_init(x0: torch.Tensor, w: torch.Tensor, eps: float, streams: int) -> torch.Tensor:
+    """fp32 [T, S, d]: every stream is rms_norm(x0) * w."""
+    e = x0 * torch.rsqrt(x0.pow(2).mean(-1, keepdim=True) + eps) * w.float()
+    return e[:, None, :].repeat(1, streams, 1).contiguous()
+
+
+def hc_step(xs: torch.Tensor, y, mix, out_w, in_w, norm_w, eps: float, act_dtype):
+    """xs fp32 [T, S, d] in place: xs[:, j] <- sum_s mix[s, j] xs[:, s] + out_w[j] y (with y); then
+    u = sum_s in_w[s] xs[:, s] (with in_w), returned normed times norm_w in ``act_dtype``, or as it is."""
+    S = xs.shape[1]
+    if y is not None:
+        xs.copy_(torch.einsum("sj,tsd->tjd", mix.float().view(S, S), xs) + out_w.float()[None, :, None] * y.float()[:, None, :])
+    if in_w is None:
+        return None
+    u = torch.einsum("s,tsd->td", in_w.float(), xs)
+    if norm_w is None:
+        return u
+    return (u * torch.rsqrt(u.pow(2).mean(-1, keepdim=True) + eps) * norm_w.float()).to(act_dtype)
+
+
+def rope_any(x: torch.Tensor, positions: torch.Tensor, dims: int, inv_freq: torch.Tensor, pairs: bool,
+             sign: float = 1.0) -> torch.Tensor:
+    """x fp32 [T, heads, D]: the first ``dims`` coordinates of each head turn by sign * position * inv_freq[i]
+    (fp64 angles), neighbours together (``pairs``) or i with i + dims / 2; the rest pass."""
+    if dims == 0:
+        return x
+    if pairs:
+        return rope_pairs(x, positions if sign > 0 else -positions, dims, inv_freq)
+    half = dims // 2
+    ang = sign * positions.double()[:, None] * inv_freq.double()[None, :]
+    c, s = torch.cos(ang).float()[:, None, :], torch.sin(ang).float()[:, None, :]
+    u, v = x[..., :half], x[..., half:dims]
+    return torch.cat([u * c - v * s, v * c + u * s, x[..., dims:]], -1)
+
+
+def rope_qkv_write(qkv: torch.Tensor, inv_freq, inv_freq_v, positions, slot_mapping, k_cache, v_cache, H: int, G: int,
+                   D: int, Dv: int, rot_dims: int, pairs: bool, v_pairs: bool) -> torch.Tensor:
+    """qkv fp32 [T, >= H D + G (D + Dv)] = q | k | v: q and k turn over their first rot_dims coordinates, v (with
+    ``inv_freq_v``) over its whole width; keys and values go to the paged planes. Returns the turned q [T, H*D]."""
+    T = qkv.shape[0]
+    q = rope_any(qkv[:, :H * D].float().view(T, H, D), positions, rot_dims, inv_freq, pairs).reshape(T, H * D)
+    if k_cache is not None:
+        k = rope_any(qkv[:, H * D:(H + G) * D].float().view(T, G, D), positions, rot_dims, inv_freq, pairs)
+        v = qkv[:, (H + G) * D:(H + G) * D + G * Dv].float().view(T, G, Dv)
+        if inv_freq_v is not None:
+            v = rope_any(v, positions, Dv, inv_freq_v, v_pairs)
+        BS = k_cache.shape[2]
+        slots = slot_mapping.long()
+        ok = slots >= 0
+        blk, off = slots[ok] // BS, slots[ok] % BS
+        k_cache[blk, :, off, :] = k[ok].to(k_cache.dtype)
+        v_cache[blk, :, off, :] = v[ok].to(v_cache.dtype)
+    return q.contiguous()
+
+
+def talk_mix(o: torch.Tensor, talk: torch.Tensor, positions, inv_freq_v, H: int, G: int, Dv: int, act_dtype,
+             v_pairs: bool) -> torch.Tensor:
+    """o fp32 [T, H * G * Dv] -> out[t, h] = sum_g talk[h, g] o[t, g, h / (H / G)], turned back by the row's position."""
+    T = o.shape[0]
+    o5 = o.float().view(T, H, G, Dv)
+    kv = torch.arange(H, device=o.device) // (H // G)
+    mixed = torch.einsum("hg,tghv->thv", talk.float().view(H, H), o5[:, :, kv, :])
+    if inv_freq_v is not None:
+        mixed = rope_any(mixed, positions, Dv, inv_freq_v, v_pairs, sign=-1.0)
+    return mixed.reshape(T, H * Dv).to(act_dtype)
+
+
+def latent_rope_write(proj: torch.Tensor, col_c: int, w, eps: float, inv_freq, positions, slot_mapping, cache, qlat,
+                      H: int, D: int, R: int, rd: int, pairs: bool) -> None:
+    """cache [blocks, 1, BS, R + rd] <- rms_norm(proj[:, col_c:+R]) * w | turned proj[:, col_c + R:+rd]; the turned
+    query parts (columns D .. D + rd - 1 of each head's block of D + rd) go to columns R .. R + rd - 1 of each head's
+    block of qlat [T, H * (R + rd)]."""
+    T = proj.shape[0]
+    if rd:
+        qr = proj[:, :H * (D + rd)].float().view(T, H, D + rd)[:, :, D:]
+        qlat.view(T, H, R + rd)[:, :, R:] = rope_any(qr, positions, rd, inv_freq, pairs)
+    if cache is None:
+        return
+    BS = cache.shape[2]
+    c = proj[:, col_c:col_c + R].float()
+    c = c * torch.rsqrt(c.pow(2).mean(-1, keepdim=True) + eps) * w.float()
+    row = [c]
+    if rd:
+        row.append(rope_any(proj[:, col_c + R:col_c + R + rd].float().view(T, 1, rd), positions, rd, inv_freq, pairs)[:, 0])
+    slots = slot_mapping.long()
+    ok = slots >= 0
+    cache[slots[ok] // BS, 0, slots[ok] % BS, :] = torch.cat(row, -1)[ok].to(cache.dtype)
+
+
+def xielu(y: torch.Tensor, ap: float, an: float, act_dtype) -> torch.Tensor:
+    z = y.float()
+    return torch.where(z > 0, ap * z * z + 0.5 * z, an * (torch.expm1(torch.clamp(z, max=0.0)) - z) + 0.5 * z).to(act_dtype)

@@ -1497,7 +1497,7 @@ LC_EXPORT int lc_attn_tile(const void* q, const void* kc, const void* vc, int ca
   if (k_ld < D || v_ld < Dv || o_col0 < 0 || o_ld < o_col0 + nvh * Dv || softcap < 0.f) return -1;
   const int NC = nvh * Dv;
   // (16-byte loads of the staged tiles: rows and column blocks start on 16-byte borders)
-  if (D % 8 || Dv % 16 || NC > 16 * kTileMaxVT || D > 256 || k_ld % 8 || v_ld % 8) return -2;
+  if (D % 8 || Dv % 8 || NC % 16 || NC > 16 * kTileMaxVT || D > 256 || k_ld % 8 || v_ld % 8) return -2;
   const int DS = D + ((4 - D % 32 + 32) % 32), VS = NC + ((16 - NC % 32 + 32) % 32);
   const size_t lds = (static_cast<size_t>(80) * DS + 16 * VS + 4 * 16 * 17) * sizeof(float);
   if (lds > 64 * 1024) return -2;

@@ -122,7 +122,7 @@ class Design:
                                     # output coordinate, ``kv_from``)
     embed_norm: bool = False        # an RMS norm (tensor ``embed.norm``) on the embedding rows
     hyper: bool = False             # the residual is ``streams`` parallel streams (tensors ``<layer>.hc<q>.{in,out,mix}``)
-    routed_ff: str = "grouped_relu2"    # "sigmoid_clamped": sigmoid scores, weight on the expert's input, clamped gated experts
+    routed_ff: str = "grouped_relu2"    # "sigmoid_clamped": sigmoid scores, weight on the expert's input, clamped gated experts | "": none
     # constants of the clamped gated unit g * sigmoid(slope g) * (u + shift)
     glu_slope: float = 1.702
     glu_shift: float = 1.0
@@ -135,7 +135,7 @@ DESIGNS: Dict[str, Design] = {
     "Surevik": Design("Surevik", ("attention",), pre_norm=True, dense_ff="", norm="dyt", tied_head=True,
                       attention="keys_as_values", routed_ff="sigmoid_clamped"),
     "Gizilorn": Design("Gizilorn", ("attention", "latent_attention"), pre_norm=True, dense_ff="xielu", attention="talking",
-                       latent="rotary", embed_norm=True, hyper=True),
+                       latent="rotary", embed_norm=True, hyper=True, routed_ff=""),
 }
 MIXERS = tuple(dict.fromkeys(m for d in DESIGNS.values() for m in d.mixers))
 
@@ -395,7 +395,7 @@ def _mlp_of(name: str, i: int, mlp: Optional[dict], design: Design):
         raise ValueError(f"{name}: layer {i}: {design.name} has no dense feed-forward")
     if kind == "dense":
         return int(mlp["ff"]), None
-    if kind != "moe" or not design.pre_norm:
+    if kind != "moe" or not design.pre_norm or not design.routed_ff:
         raise ValueError(f"{name}: layer {i}: feed-forward kind {kind!r} is not supported")
     r, g = mlp["router"], mlp["router"].get("groups") or {}
     shared = mlp.get("shared") or {}

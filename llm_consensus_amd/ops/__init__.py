@@ -1120,7 +1120,8 @@ def attn_masked(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, b
         return [(v0, min(n, G - v0), v0 * Dv) for v0 in range(0, G, n)] if n else []
     opts = (float(softcap), 1 if sink else 0)
     first = 0
-    tile_cols = max([n * Dv for n in range(1, nv + 1) if attn_tile_ok(D, n * Dv)] or [0])
+    # value heads side by side in one tile: equal groups whose width the tiles take (whole MFMA steps of 16 columns)
+    tile_cols = max([n * Dv for n in range(1, nv + 1) if nv % n == 0 and Dv % 8 == 0 and attn_tile_ok(D, n * Dv)] or [0])
     aligned = k_ld % 8 == 0 and v_ld % 8 == 0 and k_cache.data_ptr() % 16 == 0 and v_cache.data_ptr() % 16 == 0
     if n_portions > 0 and portion_rows > 0 and max_len >= ATTN_TILE_MIN_ROWS and tile_cols and aligned:
         for vh0, nvh, col0 in value_groups(tile_cols):

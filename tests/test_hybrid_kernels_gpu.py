@@ -466,3 +466,138 @@ def test_clamped_gated_experts_as_the_epilogue_of_the_packed_product(T, top, E, 
     torch.testing.assert_close(got.float().cpu(), want, atol=2e-2, rtol=2e-2)
     with pytest.raises(ValueError):
         ops.grouped_linear(x.to(DEV), src, offsets, W, torch.float32, T * top)
+
+
+# ------------------------------------------------------------------ parallel residual streams, turned values, mixed heads'
+# weights, a turned key part beside the latent row, xIELU (hybrid_streams.hip; options of the attention kernels)
+@pytest.mark.parametrize("dt", ACTS)
+@pytest.mark.parametrize("T,S,d", [(3, 1, 10), (7, 3, 72), (600, 2, 130), (5, 8, 257), (700, 4, 64)])
+def test_parallel_streams_start_and_sublayer_step(dt, T, S, d):
+    g = torch.Generator().manual_seed(T + S)
+    x0, w = torch.randn(T, d, generator=g) * 3, torch.rand(d, generator=g) + 0.5
+    xs = ops.hc_init(x0.to(DEV), w.to(DEV), 1e-3, S)
+    xr = ref.hc_init(x0, w, 1e-3, S)
+    torch.testing.assert_close(xs.cpu(), xr, atol=1e-5, rtol=1e-5)
+    xs = (xs + 0.3 * torch.randn(T, S, d, generator=g).to(DEV)).contiguous()          # streams that have grown apart
+    xr = xs.cpu().clone()
+    mix, ow, iw = torch.randn(S, S, generator=g), torch.randn(S, generator=g), torch.randn(S, generator=g)
+    nw, y = torch.rand(d, generator=g) + 0.5, torch.randn(T, d, generator=g)
+    tol = _tol(dt) if dt == torch.bfloat16 else dict(atol=2e-5, rtol=2e-5)
+    # the read alone (the first sublayer of a step), normed
+    a = ops.hc_step(xs, None, None, None, iw.to(DEV), nw.to(DEV), 1e-3, dt)
+    torch.testing.assert_close(a.float().cpu(), ref.hc_step(xr, None, None, None, iw, nw, 1e-3, dt).float(), **tol)
+    torch.testing.assert_close(xs.cpu(), xr)
+    # write and read, normed
+    a = ops.hc_step(xs, y.to(DEV), mix.to(DEV), ow.to(DEV), iw.to(DEV), nw.to(DEV), 1e-3, dt)
+    want = ref.hc_step(xr, y, mix, ow, iw, nw, 1e-3, dt)
+    torch.testing.assert_close(xs.cpu(), xr, atol=2e-5, rtol=2e-5)
+    torch.testing.assert_close(a.float().cpu(), want.float(), **tol)
+    # write, and the plain combination in fp32 (the model's output: every stream once)
+    ones = torch.ones(S)
+    u = ops.hc_step(xs, y.to(DEV), mix.to(DEV), ow.to(DEV), ones.to(DEV), None, 1e-3, None)
+    want = ref.hc_step(xr, y, mix, ow, ones, None, 1e-3, None)
+    assert u.dtype == torch.float32
+    torch.testing.assert_close(xs.cpu(), xr, atol=1e-4, rtol=1e-4)
+    torch.testing.assert_close(u.cpu(), want, atol=1e-4, rtol=1e-4)
+    torch.testing.assert_close(want, xr.sum(1), atol=1e-4, rtol=1e-4)
+    # the write alone
+    assert ops.hc_step(xs, y.to(DEV), mix.to(DEV), ow.to(DEV), None, None, 1e-3, None) is None
+    ref.hc_step(xr, y, mix, ow, None, None, 1e-3, None)
+    torch.testing.assert_close(xs.cpu(), xr, atol=1e-3, rtol=1e-4)
+
+
+@pytest.mark.parametrize("dt", ACTS)
+@pytest.mark.parametrize("H,G,D,Dv,rot,pairs,window,cap", [(4, 2, 32, 32, 8, False, 7, 3.0), (3, 3, 48, 16, 48, False, 40, 0.0), (2, 1, 16, 48, 0, False, 5, 50.0),
+                                                           (5, 1, 7, 6, 6, True, 3, 1.5), (8, 4, 16, 64, 16, False, 100, 20.0), (6, 3, 24, 200, 8, True, 30, 2.0)])
+def test_turned_values_capped_scores_a_sink_and_mixed_heads(dt, H, G, D, Dv, rot, pairs, window, cap):
+    g = torch.Generator().manual_seed(H * 100 + D)
+    lens, starts = [37, 70, 1, 1], [0, 130, 55, 3]          # two portions (one continuing at place 130), two decoded tokens
+    BSZ, MB = 16, 14
+    cu, pos, rs = _seqs(lens, starts)
+    T = int(cu[-1])
+    tables = torch.randperm(4 * MB, generator=g).to(torch.int32).view(4, MB)
+    slots = torch.tensor([int(tables[b, p // BSZ]) * BSZ + p % BSZ for b, p in zip(rs.tolist(), pos.tolist())], dtype=torch.int32)
+    qkv = torch.randn(T, H * D + G * (D + Dv) + 5, generator=g)
+    kc, vc = (torch.randn(4 * MB, G, BSZ, D, generator=g) * 0.5).to(dt), (torch.randn(4 * MB, G, BSZ, Dv, generator=g) * 0.5).to(dt)
+    inv = torch.tensor([1e3 ** (-2.0 * j / rot) for j in range(rot // 2)], dtype=torch.float64) if rot else None
+    inv_v = torch.tensor([1e3 ** (-2.0 * j / Dv) for j in range(Dv // 2)], dtype=torch.float64)
+    kd, vd = kc.clone().to(DEV), vc.clone().to(DEV)
+    q = ops.rope_qkv_write(qkv.to(DEV), inv.to(DEV) if rot else None, inv_v.to(DEV), pos.to(DEV), slots.to(DEV), kd, vd, H, G, D, Dv,
+                           rot, pairs, pairs)
+    qr = ref.rope_qkv_write(qkv, inv, inv_v, pos, slots, kc, vc, H, G, D, Dv, rot, pairs, pairs)
+    torch.testing.assert_close(q.cpu(), qr, atol=2e-5, rtol=2e-5)
+    torch.testing.assert_close(kd.float().cpu(), kc.float(), **_tol(dt))
+    torch.testing.assert_close(vd.float().cpu(), vc.float(), **_tol(dt))
+    talk = torch.eye(H) + 0.5 * torch.randn(H, H, generator=g)
+    for sink in (True, False):
+        want = ref.attn_masked(qr, kc, vc, tables, cu, pos, H, G, D, Dv, 0.2, 0, window, torch.float32, cap, sink, True)
+        assert want.shape == (T, H * G * Dv)
+        mixed = ref.talk_mix(want, talk, pos, inv_v, H, G, Dv, dt, pairs)
+        for portions, rows in ((0, 0), (2, 107)):               # the row kernel for everything; matrix-core tiles for the portions
+            got = ops.attn_masked(q, kd, vd, tables.to(DEV), cu.to(DEV), rs.to(DEV), pos.to(DEV), H, G, D, Dv, 0.2, 0, window,
+                                  torch.float32, n_portions=portions, portion_rows=rows, max_len=70, softcap=cap, sink=sink,
+                                  all_value_heads=True)
+            torch.testing.assert_close(got.cpu(), want, **(_tol(dt) if dt == torch.bfloat16 else dict(atol=2e-5, rtol=2e-5)))
+            out = ops.talk_mix(got, talk.to(DEV), pos.to(DEV), inv_v.to(DEV), H, G, Dv, dt, pairs)
+            torch.testing.assert_close(out.float().cpu(), mixed.float(), **(_tol(dt) if dt == torch.bfloat16 else dict(atol=5e-5, rtol=5e-5)))
+        # each head on its own group's values only, under the same cap and sink
+        own = ref.attn_masked(qr, kc, vc, tables, cu, pos, H, G, D, Dv, 0.2, 0, window, dt, cap, sink, False)
+        got = ops.attn_masked(q, kd, vd, tables.to(DEV), cu.to(DEV), rs.to(DEV), pos.to(DEV), H, G, D, Dv, 0.2, 0, window, dt,
+                              n_portions=2, portion_rows=107, max_len=70, softcap=cap, sink=sink)
+        torch.testing.assert_close(got.float().cpu(), own.float(), **_tol(dt))
+    # the mix alone, nothing turned back
+    no_turn = ops.talk_mix(want.to(DEV), talk.to(DEV), pos.to(DEV), None, H, G, Dv, dt)
+    torch.testing.assert_close(no_turn.float().cpu(), ref.talk_mix(want, talk, pos, None, H, G, Dv, dt, False).float(),
+                               **(_tol(dt) if dt == torch.bfloat16 else dict(atol=5e-5, rtol=5e-5)))
+
+
+@pytest.mark.parametrize("dt", ACTS)
+@pytest.mark.parametrize("H,D,R,rd,Dv,window,own", [(4, 16, 24, 8, 16, 9, True), (3, 10, 20, 6, 14, 40, True), (2, 70, 130, 80, 66, 100, False),
+                                                   (8, 64, 96, 32, 64, 33, True), (1, 5, 7, 2, 3, 4, True), (5, 8, 48, 0, 16, 12, True)])
+def test_latent_rows_with_a_turned_key_part_shared_by_the_heads(dt, H, D, R, rd, Dv, window, own):
+    g = torch.Generator().manual_seed(H * 100 + R)
+    lens, starts = [37, 70, 1, 1], [0, 130, 55, 3]
+    BSZ, MB = 16, 14
+    cu, pos, rs = _seqs(lens, starts)
+    T, W = int(cu[-1]), R + rd
+    tables = torch.randperm(4 * MB, generator=g).to(torch.int32).view(4, MB)
+    slots = torch.tensor([int(tables[b, p // BSZ]) * BSZ + p % BSZ for b, p in zip(rs.tolist(), pos.tolist())], dtype=torch.int32)
+    nq = H * (D + rd)
+    proj = torch.randn(T, nq + W + H * Dv + 3, generator=g)
+    w = torch.rand(R, generator=g) + 0.5
+    inv = torch.tensor([1e4 ** (-2.0 * j / rd) for j in range(rd // 2)], dtype=torch.float64) if rd else None
+    cache = (torch.randn(4 * MB, 1, BSZ, W, generator=g) * 0.5).to(dt)
+    cd = cache.clone().to(DEV)
+    Uk = (torch.randn(H, R, D, generator=g) / D ** 0.5).to(dt)
+    Uv = (torch.randn(H, Dv, R, generator=g) / R ** 0.5).to(dt)
+    qlat_r = torch.zeros(T, H * W)
+    ref.latent_rope_write(proj, nq, w, 1e-5, inv, pos, slots, cache if own else None, qlat_r, H, D, R, rd, True)
+    ref.head_linear(proj, Uk, torch.float32, None, D + rd, qlat_r, W)
+    qlat = torch.zeros(T, H * W, device=DEV)
+    ops.latent_rope_write(proj.to(DEV), nq, w.to(DEV), 1e-5, inv.to(DEV) if rd else None, pos.to(DEV), slots.to(DEV),
+                          cd if own else None, qlat, H, D, R, rd)
+    ops.head_linear(proj.to(DEV), Uk.to(DEV), torch.float32, x_head_stride=D + rd, out=qlat, out_head_stride=W)
+    torch.testing.assert_close(qlat.cpu(), qlat_r, atol=3e-5, rtol=3e-5)
+    torch.testing.assert_close(cd.float().cpu(), cache.float(), **_tol(dt))
+    # the cached rows are the keys; their first R columns are the values
+    want = ref.attn_masked(qlat_r, cache, cache[..., :R], tables, cu, pos, H, 1, W, R, 0.2, 0, window, torch.float32)
+    gate = proj[:, nq + W:nq + W + H * Dv]
+    o_ref = ref.head_linear(want, Uv, dt, gate, gate_full=True)
+    for portions, rows in ((0, 0), (2, 107)):
+        got = ops.attn_masked(qlat, cd, cd[..., :R], tables.to(DEV), cu.to(DEV), rs.to(DEV), pos.to(DEV), H, 1, W, R, 0.2, 0, window,
+                              torch.float32, n_portions=portions, portion_rows=rows, max_len=70)
+        torch.testing.assert_close(got.cpu(), want, **(_tol(dt) if dt == torch.bfloat16 else dict(atol=3e-5, rtol=3e-5)))
+        o = ops.head_linear(got, Uv.to(DEV), dt, gate=proj.to(DEV)[:, nq + W:nq + W + H * Dv], gate_full=True)
+        torch.testing.assert_close(o.float().cpu(), o_ref.float(), **(_tol(dt) if dt == torch.bfloat16 else dict(atol=5e-5, rtol=5e-5)))
+
+
+@pytest.mark.parametrize("dt", ACTS)
+def test_xielu(dt):
+    g = torch.Generator().manual_seed(5)
+    y = torch.randn(33, 50, generator=g) * 3
+    for ap, an in ((0.8, 1.3), (0.0, 0.5), (2.5, 4.0)):
+        got = ops.xielu(y.to(DEV)[:, 3:40], ap, an, dt)
+        z = y[:, 3:40].double()
+        want = torch.where(z > 0, ap * z * z + z / 2, an * (torch.exp(z) - 1 - z) + z / 2)
+        torch.testing.assert_close(got.float().cpu(), want.float().to(dt).float(), **_tol(dt))
+        torch.testing.assert_close(ref.xielu(y[:, 3:40], ap, an, dt).float(), got.float().cpu(), **_tol(dt))

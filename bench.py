@@ -128,10 +128,10 @@ def parse_args(argv=None):
                          "host-staged tensors (RCCL refuses two ranks on one device), model groups still use the "
                          "peer-to-peer kernels over IPC-mapped memory. Not a measurement: the ranks share the GPU")
     ap.add_argument("--hybrid", action="store_true",
-                    help="instead of the workloads: prefill / decode throughput of the hybrid decoders (Nidozen, Telurax, Surevik) beside a "
+                    help="instead of the workloads: prefill / decode throughput of the hybrid decoders (Nidozen, Telurax, Surevik, Gizilorn) beside a "
                          "Llama-shaped transformer of equal size (one GPU, random weights)")
     ap.add_argument("--hybrid-sizes", default="1k,2k", help="comma list out of 1k,2k,4k (model width)")
-    ap.add_argument("--hybrid-models", default="nidozen,llama", help="which models to run, out of surevik,telurax,nidozen,llama")
+    ap.add_argument("--hybrid-models", default="nidozen,llama", help="which models to run, out of gizilorn,surevik,telurax,nidozen,llama")
     ap.add_argument("--hybrid-phases", default="prefill,decode", help="which phases to run (for kernel profiles)")
     ap.add_argument("--hybrid-prompt", type=int, default=2048)
     ap.add_argument("--hybrid-batch", type=int, default=32)

@@ -711,6 +711,10 @@ __global__ __launch_bounds__(256) void attn_masked_kernel(
   float acc[kMaxVCols];
   int vcol[kMaxVCols], voff[kMaxVCols];            // a lane's value columns: column inside the head, row offset of the head's plane
   const int ncols = nvh * Dv;
+  if (vh0 >= 0) {                                   // blocks along z take nvh value heads each (scores are formed again: short rows)
+    vh0 += blockIdx.z * nvh;
+    o_col0 += blockIdx.z * ncols;
+  }
 #pragma unroll
   for (int i = 0; i < kMaxVCols; ++i) {
     acc[i] = 0.f;
@@ -787,7 +791,10 @@ __global__ __launch_bounds__(256) void attn_masked_kernel(
 // Row strides in LDS are padded so that the 16 rows of an operand fall into different banks.
 // The options of the row kernel (row strides, score cap, sink, value heads side by side) apply here too; the value
 // tile then holds nvh * Dv columns.
-constexpr int kTileMaxVT = 16;     // value width up to 256
+// A wave holds up to 16 accumulator tiles (256 value columns; with 32 tiles, 512 columns in one launch, the kernel ran
+// slower than two launches of 256 that each form the scores again). A block may use more than 64 KB of LDS (wide queries).
+constexpr int kTileMaxVT = 16;
+constexpr int kTileMaxLds = 160 * 1024;
 
 LC_DEVICE int lds_stride(int n, int want) { return n + ((want - n % 32 + 32) % 32); }
 
@@ -868,27 +875,37 @@ __global__ __launch_bounds__(256) void attn_tile_kernel(
   const int wave_rows = max(0, min(16, nrows - 16 * wave));
   const int wave_lo = first_key(pw0), wave_hi = pw0 + wave_rows - 1;
   // staging: a tile is 16 keys x D (x Dv) elements = 2 D (2 Dv) units of 8; a thread owns up to two of each
+  constexpr int NVU = kTileMaxVT / 8;                       // value units of 8 columns per thread (16 keys x ncols / 8 in all)
   const int ku = D / 8, vu = ncols / 8;
-  int kkey[2], kcol[2], vkey[2], vcol[2], vhead[2], vin[2];
+  int kkey[2], kcol[2], vkey[NVU], vcol[NVU], vhead[NVU], vin[NVU];
 #pragma unroll
   for (int i = 0; i < 2; ++i) {
     const int u = threadIdx.x + 256 * i;
     kkey[i] = u < 16 * ku ? u / ku : -1;
     kcol[i] = (u % ku) * 8;
+  }
+#pragma unroll
+  for (int i = 0; i < NVU; ++i) {
+    const int u = threadIdx.x + 256 * i;
     vkey[i] = u < 16 * vu ? u / vu : -1;
     vcol[i] = (u % vu) * 8;                                 // column in the tile; inside its head: vin
     vhead[i] = vh0 < 0 ? g : vh0 + vcol[i] / Dv;
     vin[i] = vcol[i] % Dv;
   }
-  Raw8<CF32> kr[2], vr[2];
+  Raw8<CF32> kr[2], vr[NVU];
   auto fetch = [&](int j0) {
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
-      const int jk = j0 + kkey[i], jv = j0 + vkey[i];
-      const bool kon = kkey[i] >= 0 && jk <= hi, von = vkey[i] >= 0 && jv <= hi;
+      const int jk = j0 + kkey[i];
+      const bool kon = kkey[i] >= 0 && jk <= hi;
       const size_t krow = kon ? (static_cast<size_t>(table[jk / BS]) * G + g) * BS + jk % BS : 0;
-      const size_t vrow = von ? (static_cast<size_t>(table[jv / BS]) * G + vhead[i]) * BS + jv % BS : 0;
       kr[i] = load_raw8<CF32>(kc, krow * k_ld + kcol[i], kon);
+    }
+#pragma unroll
+    for (int i = 0; i < NVU; ++i) {
+      const int jv = j0 + vkey[i];
+      const bool von = vkey[i] >= 0 && jv <= hi;
+      const size_t vrow = von ? (static_cast<size_t>(table[jv / BS]) * G + vhead[i]) * BS + jv % BS : 0;
       vr[i] = load_raw8<CF32>(vc, vrow * v_ld + vin[i], von);
     }
   };
@@ -907,10 +924,11 @@ __global__ __launch_bounds__(256) void attn_tile_kernel(
   for (; j0 <= hi; j0 += 16) {
     __syncthreads();                                        // the previous tile has been consumed
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
+    for (int i = 0; i < 2; ++i)
       if (kkey[i] >= 0) store_raw8<CF32>(kr[i], Ks + kkey[i] * DS + kcol[i]);
+#pragma unroll
+    for (int i = 0; i < NVU; ++i)
       if (vkey[i] >= 0) store_raw8<CF32>(vr[i], Vs + vkey[i] * VS + vcol[i]);
-    }
     __syncthreads();
     if (j0 + 16 <= hi) fetch(j0 + 16);                      // in flight while this tile is computed
     const bool mine = wave_rows > 0 && j0 <= wave_hi && j0 + 15 >= wave_lo;     // wave-uniform
@@ -1463,14 +1481,15 @@ LC_EXPORT int lc_qkv_prep(const void* qkv, int ld, const void* qn, const void* k
 LC_EXPORT int lc_attn_masked(const void* q, const void* kc, const void* vc, int cache_f32, const void* block_tables,
                              int MB, const void* row_seq, const void* positions, void* out, int act_f32, int T, int H,
                              int G, int D, int Dv, int BS, float scale, int chunk, int window, int k_ld, int v_ld,
-                             float softcap, int sink, int vh0, int nvh, int o_ld, int o_col0, hipStream_t st) {
+                             float softcap, int sink, int vh0, int nvh, int o_ld, int o_col0, int vz, hipStream_t st) {
   if (T <= 0) return 0;
-  if (H <= 0 || G <= 0 || H % G || D <= 0 || Dv <= 0 || BS <= 0 || MB <= 0) return -1;
-  if (nvh <= 0 || nvh * Dv > 64 * kMaxVCols || (vh0 < 0 && nvh != 1) || (vh0 >= 0 && vh0 + nvh > G)) return -1;
-  if (k_ld < D || v_ld < Dv || o_col0 < 0 || o_ld < o_col0 + nvh * Dv || softcap < 0.f) return -1;
+  if (H <= 0 || G <= 0 || H % G || D <= 0 || Dv <= 0 || BS <= 0 || MB <= 0 || vz <= 0 || vz > 65535) return -1;
+  // ``vz`` groups of nvh value heads each, one per block along z (vz = 1 unless value heads are named)
+  if (nvh <= 0 || nvh * Dv > 64 * kMaxVCols || (vh0 < 0 && (nvh != 1 || vz != 1)) || (vh0 >= 0 && vh0 + vz * nvh > G)) return -1;
+  if (k_ld < D || v_ld < Dv || o_col0 < 0 || o_ld < o_col0 + vz * nvh * Dv || softcap < 0.f) return -1;
   const size_t lds = 4 * static_cast<size_t>(D + 128) * sizeof(float);
   if (lds > 64 * 1024) return -1;
-  const dim3 grid(T, (H + 3) / 4), block(256);
+  const dim3 grid(T, (H + 3) / 4, vz), block(256);
 #define LC_ATT(C32, A32)                                                                                        \
   attn_masked_kernel<C32, A32><<<grid, block, lds, st>>>(                                                       \
       static_cast<const float*>(q), kc, vc, static_cast<const int32_t*>(block_tables), MB,                      \
@@ -1500,8 +1519,16 @@ LC_EXPORT int lc_attn_tile(const void* q, const void* kc, const void* vc, int ca
   if (D % 8 || Dv % 8 || NC % 16 || NC > 16 * kTileMaxVT || D > 256 || k_ld % 8 || v_ld % 8) return -2;
   const int DS = D + ((4 - D % 32 + 32) % 32), VS = NC + ((16 - NC % 32 + 32) % 32);
   const size_t lds = (static_cast<size_t>(80) * DS + 16 * VS + 4 * 16 * 17) * sizeof(float);
-  if (lds > 64 * 1024) return -2;
+  if (lds > static_cast<size_t>(kTileMaxLds)) return -2;
   const dim3 grid((max_len + 63) / 64, H, n_seq), block(256);
+  static LcDeviceOnce attr_once;
+  attr_once.run([&] {
+#define LC_TILE_ATTR(C32, A32)                                                             \
+  (void)hipFuncSetAttribute(reinterpret_cast<const void*>(attn_tile_kernel<C32, A32>),     \
+                            hipFuncAttributeMaxDynamicSharedMemorySize, kTileMaxLds)
+    LC_TILE_ATTR(true, true); LC_TILE_ATTR(true, false); LC_TILE_ATTR(false, true); LC_TILE_ATTR(false, false);
+#undef LC_TILE_ATTR
+  });
 #define LC_TILE(C32, A32)                                                                                       \
   attn_tile_kernel<C32, A32><<<grid, block, lds, st>>>(                                                         \
       static_cast<const float*>(q), kc, vc, static_cast<const int32_t*>(block_tables), MB,                      \

@@ -70,74 +70,104 @@ __global__ __launch_bounds__(256) void hc_init_kernel(const float* __restrict__ 
 // ---------------------------------------------------------------- streams: one sublayer's write, the next one's read
 // With y: xs[t, j, :] <- sum_s mix[s * S + j] xs[t, s, :] + outw[j] y[t, :] (in place: a thread owns a coordinate of
 // all streams). With inw: u = sum_s inw[s] xs[t, s, :] (of the new streams); u goes to ``u_out`` (fp32) when given,
-// and u / sqrt(mean(u^2) + eps) * normw to ``xa`` in the activation type when a norm weight is given.
-template <bool AF32, int WAVES>
+// and u / sqrt(mean(u^2) + eps) * normw to ``xa`` in the activation type when a norm weight is given. SMAX: the
+// register arrays' size (S <= SMAX). Rows of up to 8 coordinates per thread are handled in one unrolled sweep (all
+// loads in flight together, u kept in registers for the norm); wider rows loop and form u again after the reduction.
+template <int SMAX>
+struct StreamCoef {
+  const float* m;   // [S][S] from, to
+  const float* o;   // [S]
+  const float* i;   // [S]
+};
+
+template <int SMAX>
+LC_DEVICE float hc_point(float* __restrict__ xr, const float* __restrict__ yr, const StreamCoef<SMAX>& k, int S, int d, int c,
+                         bool read) {
+  float v[SMAX];
+#pragma unroll
+  for (int s = 0; s < SMAX; ++s) v[s] = s < S ? xr[static_cast<size_t>(s) * d + c] : 0.f;
+  if (yr != nullptr) {
+    const float yv = yr[c];
+    float n[SMAX];
+#pragma unroll
+    for (int j = 0; j < SMAX; ++j) {
+      float a = 0.f;
+      if (j < S) {
+#pragma unroll
+        for (int s = 0; s < SMAX; ++s)
+          if (s < S) a += k.m[s * S + j] * v[s];
+        a += k.o[j] * yv;
+        xr[static_cast<size_t>(j) * d + c] = a;
+      }
+      n[j] = a;
+    }
+#pragma unroll
+    for (int j = 0; j < SMAX; ++j) v[j] = n[j];
+  }
+  float u = 0.f;
+  if (read) {
+#pragma unroll
+    for (int s = 0; s < SMAX; ++s)
+      if (s < S) u += k.i[s] * v[s];
+  }
+  return u;
+}
+
+template <bool AF32, int WAVES, int SMAX>
 __global__ __launch_bounds__(256) void hc_step_kernel(float* __restrict__ xs, const float* __restrict__ y,
                                                       const float* __restrict__ mix, const float* __restrict__ outw,
                                                       const float* __restrict__ inw, const float* __restrict__ normw,
                                                       float eps, float* __restrict__ u_out, void* __restrict__ xa, int T,
                                                       int S, int d) {
   __shared__ float red[16];
-  __shared__ float coef[kMaxStreams * kMaxStreams + 2 * kMaxStreams];
+  __shared__ float coef[SMAX * SMAX + 2 * SMAX];
   constexpr int LANES = 64 * WAVES;
+  constexpr int UMAX = 8;
   const int row = WAVES == 1 ? blockIdx.x * 4 + (threadIdx.x >> 6) : blockIdx.x;
   const int lane = WAVES == 1 ? (threadIdx.x & 63) : threadIdx.x;
-  float* cm = coef;                                  // [S][S] from, to
-  float* co = coef + kMaxStreams * kMaxStreams;      // [S]
-  float* ci = co + kMaxStreams;                      // [S]
-  for (int i = threadIdx.x; i < S * S; i += blockDim.x) cm[i] = y != nullptr ? mix[i] : 0.f;
+  for (int i = threadIdx.x; i < S * S; i += blockDim.x) coef[i] = y != nullptr ? mix[i] : 0.f;
   for (int i = threadIdx.x; i < S; i += blockDim.x) {
-    co[i] = y != nullptr ? outw[i] : 0.f;
-    ci[i] = inw != nullptr ? inw[i] : 0.f;
+    coef[SMAX * SMAX + i] = y != nullptr ? outw[i] : 0.f;
+    coef[SMAX * SMAX + SMAX + i] = inw != nullptr ? inw[i] : 0.f;
   }
   __syncthreads();
+  const StreamCoef<SMAX> k{coef, coef + SMAX * SMAX, coef + SMAX * SMAX + SMAX};
   const bool on = WAVES != 1 || row < T;             // (idle waves still take part in the barriers)
   float* xr = xs + static_cast<size_t>(on ? row : 0) * S * d;
   const float* yr = y != nullptr ? y + static_cast<size_t>(on ? row : 0) * d : nullptr;
+  const bool read = inw != nullptr;
+  const bool fits = d <= LANES * UMAX;               // the same for every thread
   float ss = 0.f;
-  if (on)
-    for (int c = lane; c < d; c += LANES) {
-      float v[kMaxStreams];
+  float u[UMAX];
+  if (on && fits) {
 #pragma unroll
-      for (int s = 0; s < kMaxStreams; ++s) v[s] = s < S ? xr[static_cast<size_t>(s) * d + c] : 0.f;
-      if (yr != nullptr) {
-        const float yv = yr[c];
-        float n[kMaxStreams];
-#pragma unroll
-        for (int j = 0; j < kMaxStreams; ++j) {
-          float a = 0.f;
-          if (j < S) {
-#pragma unroll
-            for (int s = 0; s < kMaxStreams; ++s)
-              if (s < S) a += cm[s * S + j] * v[s];
-            a += co[j] * yv;
-            xr[static_cast<size_t>(j) * d + c] = a;
-          }
-          n[j] = a;
-        }
-#pragma unroll
-        for (int j = 0; j < kMaxStreams; ++j) v[j] = n[j];
-      }
-      if (inw != nullptr) {
-        float u = 0.f;
-#pragma unroll
-        for (int s = 0; s < kMaxStreams; ++s)
-          if (s < S) u += ci[s] * v[s];
-        ss += u * u;
-        if (u_out != nullptr) u_out[static_cast<size_t>(row) * d + c] = u;
-      }
+    for (int e = 0; e < UMAX; ++e) {
+      const int c = lane + e * LANES;
+      u[e] = c < d ? hc_point<SMAX>(xr, yr, k, S, d, c, read) : 0.f;
+      ss += u[e] * u[e];
+      if (u_out != nullptr && c < d) u_out[static_cast<size_t>(row) * d + c] = u[e];
     }
-  if (normw == nullptr || inw == nullptr) return;    // the same for every thread
+  } else if (on) {
+    for (int c = lane; c < d; c += LANES) {
+      const float uv = hc_point<SMAX>(xr, yr, k, S, d, c, read);
+      ss += uv * uv;
+      if (u_out != nullptr) u_out[static_cast<size_t>(row) * d + c] = uv;
+    }
+  }
+  if (normw == nullptr || !read) return;             // the same for every thread
   ss = WAVES == 1 ? wave_sum(ss) : block_sum(ss, red);
   if (!on) return;
   const float r = 1.f / sqrtf(ss / static_cast<float>(d) + eps);
   typename Act<AF32>::type* a = static_cast<typename Act<AF32>::type*>(xa);
-  for (int c = lane; c < d; c += LANES) {
-    float u = 0.f;                                   // the same sum in the same order as above
+  if (fits) {
 #pragma unroll
-    for (int s = 0; s < kMaxStreams; ++s)
-      if (s < S) u += ci[s] * xr[static_cast<size_t>(s) * d + c];
-    Act<AF32>::store(a, static_cast<size_t>(row) * d + c, u * r * normw[c]);
+    for (int e = 0; e < UMAX; ++e) {
+      const int c = lane + e * LANES;
+      if (c < d) Act<AF32>::store(a, static_cast<size_t>(row) * d + c, u[e] * r * normw[c]);
+    }
+  } else {
+    for (int c = lane; c < d; c += LANES)            // the same sum in the same order as above, from the new streams
+      Act<AF32>::store(a, static_cast<size_t>(row) * d + c, hc_point<SMAX>(xr, nullptr, k, S, d, c, true) * r * normw[c]);
   }
 }
 
@@ -196,26 +226,23 @@ __global__ __launch_bounds__(256) void talk_mix_kernel(const float* __restrict__
                                                        const int32_t* __restrict__ positions,
                                                        const double* __restrict__ inv_freq_v, void* __restrict__ out, int H,
                                                        int G, int Dv, int v_pairs) {
-  extern __shared__ float lds_tm[];                // mixed [H*Dv], then cos / sin [Dv]
-  const int t = blockIdx.x;
+  extern __shared__ float lds_tm[];                // mixed [Dv], then cos / sin [Dv]
+  const int t = blockIdx.x, h = blockIdx.y;        // a block per (token, head)
   float* mixed = lds_tm;
-  float* cs = lds_tm + H * Dv;
+  float* cs = lds_tm + Dv;
   if (inv_freq_v != nullptr) angle_table(cs, Dv >> 1, static_cast<double>(positions[t]), inv_freq_v);
-  const float* ot = o + static_cast<size_t>(t) * H * G * Dv;
-  const int rep = H / G;
-  for (int i = threadIdx.x; i < H * Dv; i += blockDim.x) {
-    const int h = i / Dv, c = i - h * Dv;
-    const int kv = h / rep;
+  const int kv = h / (H / G);
+  const float* ot = o + (static_cast<size_t>(t) * H * G + kv) * Dv;
+  for (int c = threadIdx.x; c < Dv; c += blockDim.x) {
     float a = 0.f;
-    for (int g = 0; g < H; ++g) a += talk[h * H + g] * ot[(static_cast<size_t>(g) * G + kv) * Dv + c];
-    mixed[i] = a;
+    for (int g = 0; g < H; ++g) a += talk[h * H + g] * ot[static_cast<size_t>(g) * G * Dv + c];
+    mixed[c] = a;
   }
   __syncthreads();
   typename Act<AF32>::type* dst = static_cast<typename Act<AF32>::type*>(out);
-  for (int i = threadIdx.x; i < H * Dv; i += blockDim.x) {
-    const int c = i % Dv;
-    const float r = inv_freq_v != nullptr ? turned(mixed + i - c, c, Dv, cs, v_pairs, -1.f) : mixed[i];
-    Act<AF32>::store(dst, static_cast<size_t>(t) * H * Dv + i, r);
+  for (int c = threadIdx.x; c < Dv; c += blockDim.x) {
+    const float r = inv_freq_v != nullptr ? turned(mixed, c, Dv, cs, v_pairs, -1.f) : mixed[c];
+    Act<AF32>::store(dst, (static_cast<size_t>(t) * H + h) * Dv + c, r);
   }
 }
 
@@ -294,15 +321,20 @@ LC_EXPORT int lc_hc_step(void* xs, const void* y, const void* mix, const void* o
   if (u_out != nullptr && inw == nullptr) return -1;
   const bool few = T <= 512;
   const dim3 grid(few ? T : (T + 3) / 4), block(256);
-#define LC_HC(A32, WAVES)                                                                                          \
-  hc_step_kernel<A32, WAVES><<<grid, block, 0, st>>>(                                                              \
+#define LC_HC(A32, WAVES, SMAX)                                                                                    \
+  hc_step_kernel<A32, WAVES, SMAX><<<grid, block, 0, st>>>(                                                        \
       static_cast<float*>(xs), static_cast<const float*>(y), static_cast<const float*>(mix),                       \
       static_cast<const float*>(outw), static_cast<const float*>(inw), static_cast<const float*>(normw), eps,      \
       static_cast<float*>(u_out), xa, T, S, d)
-  if (act_f32 && few) LC_HC(true, 4);
-  else if (act_f32) LC_HC(true, 1);
-  else if (few) LC_HC(false, 4);
-  else LC_HC(false, 1);
+#define LC_HC_S(A32, WAVES)               \
+  if (S <= 2) LC_HC(A32, WAVES, 2);       \
+  else if (S <= 4) LC_HC(A32, WAVES, 4);  \
+  else LC_HC(A32, WAVES, kMaxStreams)
+  if (act_f32 && few) { LC_HC_S(true, 4); }
+  else if (act_f32) { LC_HC_S(true, 1); }
+  else if (few) { LC_HC_S(false, 4); }
+  else { LC_HC_S(false, 1); }
+#undef LC_HC_S
 #undef LC_HC
   LC_RETURN_LAST_ERROR();
 }
@@ -333,10 +365,11 @@ LC_EXPORT int lc_talk_mix(const void* o, const void* talk, const void* positions
   if (T <= 0) return 0;
   if (H <= 0 || G <= 0 || H % G || Dv <= 0 || o == nullptr || talk == nullptr || out == nullptr) return -1;
   if (inv_freq_v != nullptr && ((Dv & 1) || positions == nullptr)) return -1;
-  const size_t lds = static_cast<size_t>(H * Dv + Dv + 1) * sizeof(float);
-  if (lds > 64 * 1024) return -1;
+  const size_t lds = static_cast<size_t>(2 * Dv + 1) * sizeof(float);
+  if (lds > 64 * 1024 || H > 65535) return -1;
+  const int threads = Dv <= 64 ? 64 : (Dv <= 128 ? 128 : 256);
 #define LC_TM(A32)                                                                                               \
-  talk_mix_kernel<A32><<<dim3(T), dim3(256), lds, st>>>(static_cast<const float*>(o), static_cast<const float*>(talk), \
+  talk_mix_kernel<A32><<<dim3(T, H), dim3(threads), lds, st>>>(static_cast<const float*>(o), static_cast<const float*>(talk), \
                                                         static_cast<const int32_t*>(positions),                  \
                                                         static_cast<const double*>(inv_freq_v), out, H, G, Dv, v_pairs)
   if (act_f32) LC_TM(true);

@@ -1,6 +1,6 @@
-"""Prefill and decode throughput of the hybrid decoders (Nidozen, Telurax, Surevik) beside each other and a
+"""Prefill and decode throughput of the hybrid decoders (Nidozen, Telurax, Surevik, Gizilorn) beside each other and a
 Llama-shaped transformer of equal width, depth and head sizes (``bench.py --hybrid``,
-``--hybrid-models surevik,telurax,nidozen,llama``). Random weights, synthetic tokens.
+``--hybrid-models gizilorn,surevik,telurax,nidozen,llama``). Random weights, synthetic tokens.
 
 Per size: one prompt of ``prompt`` tokens goes through each engine as a single step (prefill
 tokens/s), then ``batch`` requests decode ``new`` tokens each from recorded steps (decode tokens/s).
@@ -11,7 +11,10 @@ sixteenth of the dense width plus 4 identity experts in 4 groups of which 2 are 
 expert of a quarter); the Surevik stack is window attention (the window is the others' chunk) with a routed
 feed-forward of the same sizes in every layer (32 clamped gated experts of a sixteenth of the dense width, 4
 chosen, a gated shared expert of a quarter), its second and third layer run twice, so that it has as many
-layer runs as the others have layers; the transformer has full causal attention and a SwiGLU feed-forward. Prints one
+layer runs as the others have layers; the Gizilorn stack repeats (attention with mixed heads' weights, the same,
+latent attention with rows of its own, latent attention on those rows) over two residual streams, windows of the
+others' chunk, compressed rows of width 128 beside a turned key part of 64, a dense xIELU feed-forward in every
+layer; the transformer has full causal attention and a SwiGLU feed-forward. Prints one
 JSON line. Per-kernel times come from running this under ``rocprofv3 --kernel-trace --stats``.
 """
 from __future__ import annotations
@@ -91,6 +94,30 @@ def surevik_config(s: dict):
                             name="surevik-bench")
 
 
+def gizilorn_config(s: dict):
+    from .models.hybrid import config_from_dict
+
+    ff = {"kind": "dense", "ff": s["ff"]}
+    attn = {"type": "attention",
+            "mixer": {"heads": s["heads"], "kv_heads": s["kv"], "dim": s["dim"], "vdim": s["dim"], "scale": s["dim"] ** -0.5,
+                      "softcap": 50.0, "mask": {"size": s["chunk"]}, "rot": {"dims": s["dim"] // 2, "base": 10000.0}}, "mlp": ff}
+
+    def latent(kv_from=None):
+        m = {"heads": s["heads"], "dim": s["dim"], "rot_dim": 64, "vdim": s["dim"], "kv_rank": 128,
+             "scale": (s["dim"] + 64) ** -0.5, "mask": {"size": s["chunk"]}, "rot": {"dims": 64, "base": 1e6}}
+        if kv_from is not None:
+            m["kv_from"] = kv_from
+        return {"type": "latent_attention", "mixer": m, "mlp": ff}
+    layers = []
+    for i in range(s["layers"]):
+        k = i % 4
+        if k == 2:
+            own = i
+        layers.append(attn if k < 2 else latent(None if k == 2 else own))
+    return config_from_dict({"architecture": "Gizilorn", "vocab": s["vocab"], "width": s["width"], "norm": {"eps": 1e-5},
+                             "streams": 2, "layers": layers}, name="gizilorn-bench")
+
+
 def transformer_config(s: dict):
     from .models.config import ModelConfig
 
@@ -162,6 +189,8 @@ def run(a) -> int:
                 model = HybridModel.random_init(telurax_config(s), dev, seed=1)
             elif kind == "surevik":
                 model = HybridModel.random_init(surevik_config(s), dev, seed=1)
+            elif kind == "gizilorn":
+                model = HybridModel.random_init(gizilorn_config(s), dev, seed=1)
             else:
                 model = TransformerModel.random_init(transformer_config(s), dev, seed=1)
             row[kind] = _measure(model, a.hybrid_prompt, a.hybrid_batch, a.hybrid_new, a.steps, a.warmup, phases)
@@ -172,7 +201,8 @@ def run(a) -> int:
             k = ph + "_tokens_per_s"
             if all(k in row.get(m, {}) for m in ("nidozen", "llama")):
                 row[ph + "_ratio"] = row["nidozen"][k] / row["llama"][k]
-            for mine, others in (("telurax", ("nidozen", "llama")), ("surevik", ("telurax", "nidozen", "llama"))):
+            for mine, others in (("telurax", ("nidozen", "llama")), ("surevik", ("telurax", "nidozen", "llama")),
+                                 ("gizilorn", ("surevik", "telurax", "nidozen", "llama"))):
                 for other in others:
                     if all(k in row.get(m, {}) for m in (mine, other)):
                         row[f"{ph}_{mine}_over_{other}"] = row[mine][k] / row[other][k]

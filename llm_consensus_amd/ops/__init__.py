@@ -1058,11 +1058,12 @@ def qkv_prep(qkv: torch.Tensor, q_norm: torch.Tensor, k_norm: Optional[torch.Ten
 
 def attn_tile_ok(D: int, Dv: int) -> bool:
     """Whether prompt portions of these head widths take the matrix-core kernel (fp32 MFMA tiles:
-    widths in whole MFMA steps, one block's tiles within 64 KB of LDS); otherwise the row kernel."""
+    widths in whole MFMA steps, up to 256 value columns, one block's tiles within 160 KB of LDS);
+    otherwise the row kernel."""
     if D % 8 or Dv % 16 or Dv > 256 or D > 256:
         return False
     ds, vs = D + ((4 - D % 32 + 32) % 32), Dv + ((16 - Dv % 32 + 32) % 32)
-    return (80 * ds + 16 * vs + 4 * 16 * 17) * 4 <= 64 * 1024
+    return (80 * ds + 16 * vs + 4 * 16 * 17) * 4 <= 160 * 1024
 
 
 ATTN_TILE_MIN_ROWS = int(os.environ.get("LC_ATTN_TILE_MIN_ROWS", "16"))
@@ -1130,14 +1131,13 @@ def attn_masked(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, b
                         D, Dv, BS, float(scale), int(chunk), int(window), k_ld, v_ld, *opts, vh0, nvh, o_ld, col0)
         first = portion_rows
     if first < T:
-        groups = value_groups(512)
-        if not groups:
+        if Dv > 512:
             raise ValueError("attn_masked: the row kernel takes value widths up to 512")
-        for vh0, nvh, col0 in groups:
-            _hip().call("lc_attn_masked", q[first:].data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), cf,
-                        block_tables.data_ptr(), MB, row_seq[first:].data_ptr(), positions[first:].data_ptr(),
-                        out[first:].data_ptr(), af, T - first, H, G, D, Dv, BS, float(scale), int(chunk), int(window),
-                        k_ld, v_ld, *opts, vh0, nvh, o_ld, col0)
+        # (value heads side by side: a block along z per value head; the short rows' scores are formed again there)
+        _hip().call("lc_attn_masked", q[first:].data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), cf,
+                    block_tables.data_ptr(), MB, row_seq[first:].data_ptr(), positions[first:].data_ptr(),
+                    out[first:].data_ptr(), af, T - first, H, G, D, Dv, BS, float(scale), int(chunk), int(window),
+                    k_ld, v_ld, *opts, 0 if all_value_heads else -1, 1, o_ld, 0, nv)
     return out
 
 

@@ -68,7 +68,7 @@ _SIGNATURES = {
     "lc_headnorm_gate": [_P, _P, _P, _I, _P, _I, _I, _I, _I, _F, _I, _I, _I, _P, _P],
     "lc_qkv_prep": [_P, _I, _P, _P, _P, _P, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _F, _I, _P],
     "lc_attn_masked": [_P, _P, _P, _I, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _I, _I,
-                       _I, _I, _F, _I, _I, _I, _I, _I, _P],
+                       _I, _I, _F, _I, _I, _I, _I, _I, _I, _P],
     "lc_attn_tile": [_P, _P, _P, _I, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _F, _I, _I,
                      _I, _I, _F, _I, _I, _I, _I, _I, _P],
     "lc_gemm_any": [_P, _I, _I, _P, _I, _P, _P, _I, _I, _I, _I, _I, _P],

@@ -436,7 +436,8 @@ def config_from_dict(c: dict, name: str = "hybrid", tensor_shapes: Optional[Dict
         elif t == "attention" and design.attention == "talking":
             mask, rot = m.get("mask") or {}, m.get("rot") or {}
             layers.append(LayerSpec(t, heads=int(m["heads"]), kv_heads=int(m.get("kv_heads", m["heads"])),
-                                    dim=int(m["dim"]), vdim=int(m.get("vdim", m["dim"])), scale=float(m["scale"]),
+                                    dim=int(m["dim"]), vdim=int(m.get("vdim", m["dim"])),
+                                    scale=float(m.get("scale", int(m["dim"]) ** -0.5)),
                                     window=int(mask.get("size", 0)), rot_dims=int(rot.get("dims", 0)),
                                     rot_base=float(rot.get("base", 10000.0)), talk=True, softcap=float(m.get("softcap", 0.0)),
                                     sink=True, rotate_values=True, ff=ff))
@@ -444,7 +445,8 @@ def config_from_dict(c: dict, name: str = "hybrid", tensor_shapes: Optional[Dict
             mask, rot = m.get("mask") or {}, m.get("rot") or {}
             kvf = m.get("kv_from")
             layers.append(LayerSpec(t, heads=int(m["heads"]), dim=int(m["dim"]), vdim=int(m.get("vdim", m["dim"])),
-                                    kv_rank=int(m["kv_rank"]), rot_dim=int(m.get("rot_dim", 0)), scale=float(m["scale"]),
+                                    kv_rank=int(m["kv_rank"]), rot_dim=int(m.get("rot_dim", 0)),
+                                    scale=float(m.get("scale", (int(m["dim"]) + int(m.get("rot_dim", 0))) ** -0.5)),
                                     window=int(mask.get("size", 0)), rot_dims=int(rot.get("dims", m.get("rot_dim", 0))),
                                     rot_base=float(rot.get("base", 10000.0)), kv_from=-1 if kvf is None else int(kvf),
                                     gate_full=True, ff=ff))

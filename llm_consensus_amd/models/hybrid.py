@@ -14,8 +14,8 @@ Gizilorn (pre-norm, a residual of several parallel streams):
   output is ``head . rms_norm(sum_s x_s)``;
 * ``attention``: biased q / k / v projections; q and k turn over their first ``rot.dims`` coordinates (i with
   i + dims / 2), the values over their WHOLE width by their own position and are cached so; scores are scaled,
-  then capped (``softcap * tanh(s / softcap)``); a window of ``mask.size`` positions; a softmax with one added to
-  its denominator; the heads' weights are mixed by ``talk`` [H, H] before they meet the values of the head's own
+  then capped (``softcap * tanh(s / softcap)``); a window of ``mask.size`` positions; a softmax whose denominator carries
+  an extra 1 (a sink); the heads' weights are mixed by ``talk`` [H, H] before they meet the values of the head's own
   group; each head's result turns back by the row's position; ``W_o``;
 * ``latent_attention``: a query head is [dim plain | rot_dim turned] coordinates; the cached row per token is the
   RMS-normed compressed row (``kv_rank``) beside ONE turned key part (``rot_dim``, neighbouring pairs) that all
@@ -188,7 +188,7 @@ class LayerSpec:
     rot_base: float = 10000.0
     kv_from: int = -1            # attention / latent attention: read this layer's cached rows (-1: own)
     values_are_keys: bool = False    # attention: no norms, biases or value projection; neighbouring rotary pairs
-    # attention whose heads' weights are mixed: score cap (0: none), a softmax with one added to its denominator,
+    # attention whose heads' weights are mixed: score cap (0: none), a softmax whose denominator carries an extra 1,
     # values turned by their own position over their whole width (and the result turned back)
     talk: bool = False
     softcap: float = 0.0

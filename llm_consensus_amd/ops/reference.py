@@ -405,7 +405,7 @@ def attn_masked(q: torch.Tensor, k_cache, v_cache, block_tables, cu_q, positions
     """q fp32 [T, H*D]; paged keys [blocks, G, BS, D] and values [blocks, G, BS, Dv]. The row at
     position p sees keys j <= p with j >= floor(p / chunk) * chunk (``chunk`` > 0) and
     j > p - window (``window`` > 0). Scores, softmax and the weighted sum in fp32. ``softcap`` > 0: scores
-    become softcap * tanh(score / softcap); ``sink``: one is added to the softmax's denominator (an entry of
+    become softcap * tanh(score / softcap); ``sink``: the softmax's denominator carries an extra 1 (an entry of
     score 0 without a value); ``all_value_heads``: every head's weights meet the values of all G value heads,
     result [T, H * G * Dv]."""
     T = q.shape[0]

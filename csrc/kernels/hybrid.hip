@@ -8,6 +8,8 @@
 // Pre-norm designs add: a residual step fused with a per-coordinate RMS norm or with a Dynamic Tanh
 // norm, latent attention's cached row, matrix memories, per-head products, gated units (plain and
 // clamped), and attention whose values are its keys before they rotate in neighbouring pairs.
+// The two attention kernels take options that further designs combine: row strides of the planes (values that are a
+// column block of the key rows), a cap on the scores, a sink in the softmax, several value heads under one head's weights.
 //
 // A step's sequences are described by cu_q [B+1] (row ranges), positions [T] and slots [B]
 // (state slot of the sequence; < 0: padding row of a recorded step, skipped). A sequence whose
